@@ -15,6 +15,9 @@ the SAME page and slot bookkeeping:
   * sink-attention layers (grouped-query softmax attention whose values
     are the raw key projection): the dense page layout, k_cache[i] holding
     normed+rotated keys and v_cache[i] the keys as projected;
+  * head-mixing attention layers: the same two pools, k_cache[i] holding
+    rotated unit-norm keys, v_cache[i] the value projection; a layer that
+    runs several times (a repeated block) has pools per run;
   * linear-attention / retention / delta-rule layers: no pages, a recurrent
     state [n_slots, heads, dim, vdim] fp32 per sequence slot;
   * every layer with a convolution: the last taps-1 conv inputs
@@ -107,7 +110,7 @@ class PagedKV:
                 if m.kind == "latent_attention":
                     k = torch.zeros(self.n_blocks, self.block_size,
                                     m.cache_dim, device=dev, dtype=self.dtype)
-                elif m.kind == "sink_attention":
+                elif m.kind in ("sink_attention", "talk_attention"):
                     # the dense models' page layout: one (key, head) row
                     # contiguous; values here are the raw key projection
                     k = torch.zeros(self.n_blocks, m.kv_heads,

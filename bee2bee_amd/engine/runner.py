@@ -89,6 +89,13 @@ class Runner:
         return ops.fused_add_rmsnorm(x, resid, w, self.spec.rms_eps)
 
     def lm_head(self, hidden: torch.Tensor) -> torch.Tensor:
+        if self.spec.is_hybrid and self.spec.norm_type == "group_rmsnorm":
+            # fp32 residual stream, weighted grouped final norm
+            normed = ops.add_group_rmsnorm(
+                hidden.contiguous(), None, None, None,
+                self.weights.final_norm, self.spec.norm_groups,
+                self.spec.rms_eps, self.dtype)
+            return F.linear(normed, self.weights.lm_head)
         if self.spec.is_hybrid and self.weights.final_gain is None:
             # fp32 residual stream, weighted final norm
             normed = ops.rmsnorm_f32(
@@ -204,15 +211,18 @@ class Runner:
         per-expert gather/GEMM/scatter for prefill-sized ones.
 
         ffn (models/hybrid.py MoEFFNSpec) overrides the uniform-stack
-        sizes per layer, routes on fp32 logits and swaps the activation for
-        the clamped GLU; routing (top-k, softmax over the chosen logits) and
-        the three execution strategies are shared."""
+        sizes per layer, routes on fp32 logits and applies the layer's
+        activation (clamped GLU or silu GLU) and scoring rule (softmax over
+        the chosen logits, or softmax over all experts with a group-limited
+        choice); the three execution strategies are shared."""
         s = self.spec
         if ffn is not None:
             E, I, top_k = ffn.n_experts, ffn.ff, ffn.top_k
             logits = F.linear(x.float(), lw.moe_gate)
 
             def act_fn(gu):
+                if ffn.act == "silu_glu":
+                    return ops.silu_glu(gu)
                 return ops.clamped_glu(gu, ffn.limit, ffn.alpha)
         else:
             E, I, top_k = s.n_experts, s.intermediate_size, s.top_k_experts
@@ -228,7 +238,12 @@ class Runner:
             return self.ep.forward(x, lw.moe_gate, w_gu, w_dn)
         if ffn is None:
             logits = F.linear(x, lw.moe_gate)
-        weights, idx = ops.moe_topk_gate(logits, top_k)  # [T,k]
+        if ffn is not None and ffn.score == "softmax_all":
+            # scores over all experts, group-limited choice, no renorm
+            weights, idx = ops.group_topk_gate(logits, top_k, ffn.n_groups,
+                                               ffn.keep_groups)
+        else:
+            weights, idx = ops.moe_topk_gate(logits, top_k)  # [T,k]
         T, H = x.shape
 
         if T <= self.MOE_DENSE_MAX_TOKENS:
@@ -408,14 +423,22 @@ class Runner:
 
     # --------------------------------------------------------- hybrid stacks
 
-    def _rope_tables(self, dims: int, base: float, f64: bool = False):
-        """cos/sin tables per (dims, base); f64: angles evaluated in float64
-        before the single rounding to fp32."""
-        key = (dims, base, f64)
+    def _rope_tables(self, dims: int, base: float, f64: bool = False,
+                     scaling=None):
+        """cos/sin tables per (dims, base[, scaling]); f64: angles evaluated
+        in float64 before the single rounding to fp32. scaling: the
+        wavelength-dependent frequency scaling {factor, original, fast,
+        slow} (always float64 angles)."""
+        key = (dims, base, f64,
+               tuple(sorted(scaling.items())) if scaling else None)
         t = self._rope_by_cfg.get(key)
         if t is None:
-            make = ops.rope_tables_f64 if f64 else ops.rope_tables
-            t = make(self.spec.max_seq_len, dims, base, self.device)
+            if scaling:
+                t = ops.rope_tables_scaled(self.spec.max_seq_len, dims, base,
+                                           scaling, self.device)
+            else:
+                make = ops.rope_tables_f64 if f64 else ops.rope_tables
+                t = make(self.spec.max_seq_len, dims, base, self.device)
             self._rope_by_cfg[key] = t
         return t
 
@@ -453,6 +476,8 @@ class Runner:
         if s.embed_scale != 1.0:
             x = x * s.embed_scale
         n = s.n_layers
+        if s.layer_specs[0].form == "sandwich_w":
+            return self._forward_sandwich_w(x, meta)
         if s.layer_specs[0].form == "parallel":
             # x += mixer(h) + ffn(h), h = unit(x) * w: the residual add and
             # the next layer's norm run as one kernel
@@ -532,6 +557,85 @@ class Runner:
                           lw.w_down)
         return ops.add_scalar_rmsnorm(x, y, lw.gains[3], next_gain, eps, dt,
                                       y2=y2)
+
+    # ---------------------------------------------- weighted-sandwich layers
+
+    def _forward_sandwich_w(self, x: torch.Tensor, meta) -> torch.Tensor:
+        """x += w1b * gnorm(mixer(w1 * gnorm(x))); x += w2b * gnorm(ffn(w2 *
+        gnorm(x))) with grouped RMS norms; a layer run with `step_row` adds
+        that row of the step table to the residual first. Post-norm,
+        residual add, step add and the next pre-norm are ONE kernel. The
+        layer list is the list of RUNS: a repeated block appears once per
+        pass, sharing weights (LayerSpec.weights_of) but not pages."""
+        s, W = self.spec, self.weights
+        G, eps, dt = s.norm_groups, s.rms_eps, self.dtype
+        n = s.n_layers
+
+        def step_of(i):
+            r = s.layer_specs[i].step_row if i < n else None
+            return None if r is None else W.step_table[r]
+
+        normed = ops.add_group_rmsnorm(x, None, None, step_of(0),
+                                       W.layers[0].norms[0], G, eps, dt)
+        for i in range(n):
+            lw, l = W.layers[i], s.layer_specs[i]
+            y = self._talk_attn_part(i, l.mixer, lw, normed, meta)
+            nxt_w = W.layers[i + 1].norms[0] if i + 1 < n else None
+            nxt_step = step_of(i + 1)
+            tap = self.layer_tap is not None
+            f = l.ffn
+            if f is not None:
+                normed = ops.add_group_rmsnorm(x, y, lw.norms[1], None,
+                                               lw.norms[2], G, eps, dt)
+                if getattr(f, "n_experts", 0):
+                    y = self._moe_mlp(lw, normed, ffn=f)
+                else:
+                    z = F.linear(normed, lw.w_gate_up)
+                    y = F.linear(ops.polynorm(z, lw.act_coef, eps, dt),
+                                 lw.w_down)
+                post = lw.norms[3]
+            else:
+                post = lw.norms[1]
+            if tap:
+                # the probe sees the residual before the next run's step
+                ops.add_group_rmsnorm(x, y, post, None, None, G, eps, dt)
+                self.layer_tap(i, x)
+                normed = (ops.add_group_rmsnorm(x, None, None, nxt_step,
+                                                nxt_w, G, eps, dt)
+                          if nxt_w is not None else None)
+            else:
+                normed = ops.add_group_rmsnorm(x, y, post, nxt_step, nxt_w,
+                                               G, eps, dt)
+        return x
+
+    def _talk_attn_part(self, i: int, m, lw, h: torch.Tensor,
+                        meta) -> torch.Tensor:
+        """Head-mixing windowed attention of layer run i on the normed
+        input h: one fused projection [q | k | v | gate]; rotation, unit
+        norm and page store in one kernel; attention + head mixing + gate;
+        output projection."""
+        (positions, slot_mapping, cu, seq_idx, block_table, _,
+         max_qlen) = meta
+        T = h.shape[0]
+        proj = F.linear(h, lw.wqkv)
+        nq, nk, nv = m.heads * m.dim, m.kv_heads * m.dim, m.kv_heads * m.vdim
+        q = proj[:, :nq].view(T, m.heads, m.dim)
+        k = proj[:, nq : nq + nk].view(T, m.kv_heads, m.dim)
+        v = proj[:, nq + nk : nq + nk + nv].view(T, m.kv_heads, m.vdim)
+        gate = proj[:, nq + nk + nv :]
+        cos = sin = None
+        if m.rope_dims:
+            cos, sin = self._rope_tables(m.rope_dims, m.rope_base, f64=True,
+                                         scaling=m.rope_scaling)
+        k_cache, v_cache = self.kv.k_cache[i], self.kv.v_cache[i]
+        # q leaves this rotated, unit-norm and times the score scale
+        ops.rope_unit_store(q, k, v, self.spec.rms_eps, m.rope_dims,
+                            positions, cos, sin, m.scale, k_cache, v_cache,
+                            slot_mapping)
+        out = torch.empty(T, m.out_size, dtype=self.dtype, device=h.device)
+        ops.talk_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
+                      cu, lw.talk, gate, m.window, out, max_qlen)
+        return F.linear(out, lw.wo)
 
     # ------------------------------------------------- parallel-form layers
 

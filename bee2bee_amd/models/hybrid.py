@@ -22,6 +22,16 @@ output feeds the mixer AND the feed-forward, both added to the residual):
   layers[i].mixer.{heads, kv_heads, dim, vdim, decay, conv, rot.{base,dims},
   scale, left, right, left_scale, right_scale},
   layers[i].mlp.{kind: dense, ff} (or null).
+
+Pimodra config.json keys (weighted grouped RMS norms before and after each
+sublayer; a block of layers may run several times with the same tensors):
+  architecture, vocab, width, norm.{eps, groups},
+  loop.{start, stop, times} (or absent),
+  layers[i].type = attention,
+  layers[i].mixer.{heads, kv_heads, dim, vdim, scale, mask.size,
+  rot.{base, dims, scaling.{factor, original, fast, slow}}},
+  layers[i].mlp.{kind: dense, ff} | {kind: moe, expert.ff,
+  router.{experts, top, groups.{count, keep}}} (or null).
 """
 from __future__ import annotations
 
@@ -164,6 +174,42 @@ class SinkAttnSpec:
 
 
 @dataclass
+class TalkAttnSpec:
+    """Grouped-query softmax attention over paged keys and values with a
+    sliding window, whose per-head softmax weights are MIXED across heads
+    before they meet the values: w'_h = sum_g talk[h, g] w_g, and head h
+    applies w'_h to the values of its own key/value head. Queries and keys
+    are rotated (first rope_dims coordinates, pairs (i, i + rope_dims/2),
+    optionally with a wavelength-dependent frequency scaling) and THEN made
+    unit-RMS per head without a weight. The concatenated heads are gated by
+    sigmoid of a projection of the mixer input before the output
+    projection. window: 0 = every earlier position, else 0 <= i - j < window.
+    rope_scaling: None or {factor, original, fast, slow}."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0
+    rope_base: float = 10000.0
+    rope_dims: int = 0
+    rope_scaling: Optional[Dict[str, float]] = None
+
+    kind = "talk_attention"
+
+    @property
+    def in_sizes(self) -> Tuple[Tuple[str, int], ...]:
+        """Rows of the fused input projection, in order."""
+        return (("q", self.heads * self.dim), ("k", self.kv_heads * self.dim),
+                ("v", self.kv_heads * self.vdim),
+                ("g", self.heads * self.vdim))
+
+    @property
+    def out_size(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclass
 class ParallelMixerSpec:
     """Two mixers on the same input, summed with fixed scales."""
     left: Any               # SinkAttnSpec
@@ -184,7 +230,9 @@ class ParallelMixerSpec:
 
 @dataclass
 class DenseFFNSpec:
-    """down(act(up h)); act "relu2" is the square of relu."""
+    """down(act(up h)); act "relu2" is the square of relu; "polynorm" is
+    a unit(z) + b unit(z^2) + c unit(z^3) + e with four learned numbers
+    (powers element by element, unit over the ff axis)."""
     ff: int
     act: str = "relu2"
 
@@ -193,14 +241,25 @@ class DenseFFNSpec:
 class MoEFFNSpec:
     """Routed experts (+ optional always-on shared expert) with the clamped
     GLU activation: g = min(gate, limit), u = clamp(up, +-limit),
-    y = g * sigmoid(alpha g) * (u + 1)."""
+    y = g * sigmoid(alpha g) * (u + 1).
+    act "silu_glu": y = silu(gate) * up instead.
+    score "softmax_topk": top-k on the logits, weights = softmax over the
+    chosen logits. score "softmax_all": scores = softmax over ALL experts,
+    the top-k scores are the weights as they are (no renormalization); with
+    n_groups > 1 the experts form equal groups of neighbours, a group's
+    score is its largest expert score, and only experts of the best
+    keep_groups groups can be chosen."""
     n_experts: int
     top_k: int
     ff: int
-    limit: float
+    limit: float = 0.0
     shared_ff: int = 0
     shared_limit: float = 0.0
     alpha: float = 1.702
+    act: str = "clamped_glu"
+    score: str = "softmax_topk"
+    n_groups: int = 1
+    keep_groups: int = 1
 
 
 @dataclass
@@ -209,9 +268,15 @@ class LayerSpec:
     ffn: Any = None                 # MoEFFNSpec | DenseFFNSpec | None
     # "sandwich": scalar-gain norms before and after each sublayer, mixer
     # then feed-forward. "parallel": x += mixer(h) + ffn(h), h = norm(x) * w.
+    # "sandwich_w": as "sandwich" with weighted, grouped RMS norms.
     form: str = "sandwich"
     # layer whose tensors this layer uses (its own cache and state)
     weights_of: Optional[int] = None
+    # row of the model's step table added to the residual right before
+    # this layer (the first layer of a pass over a repeated block)
+    step_row: Optional[int] = None
+    # index of the checkpoint layer ('l<src>.') this run executes
+    src: Optional[int] = None
 
     @property
     def kind(self) -> str:
@@ -327,6 +392,81 @@ def parallel_layer_specs_from_cfg(layers: List[Dict[str, Any]]
     return out
 
 
+def _talk_attn_from_cfg(m: Dict[str, Any]) -> TalkAttnSpec:
+    heads = int(m["heads"])
+    kv_heads = int(m.get("kv_heads", heads))
+    if heads % kv_heads:
+        raise ValueError("attention: heads must be a multiple of kv_heads")
+    rot = m.get("rot") or {}
+    dims = int(rot.get("dims", 0))
+    if dims % 2 or dims > int(m["dim"]):
+        raise ValueError("attention: rot.dims must be even and <= dim")
+    sc = rot.get("scaling") or None
+    if sc is not None:
+        sc = {k: float(sc[k]) for k in ("factor", "original", "fast", "slow")}
+    return TalkAttnSpec(
+        heads=heads, kv_heads=kv_heads, dim=int(m["dim"]),
+        vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+        window=int((m.get("mask") or {}).get("size", 0) or 0),
+        rope_base=float(rot.get("base", 10000.0)), rope_dims=dims,
+        rope_scaling=sc)
+
+
+def _pimodra_ffn_from_cfg(f: Optional[Dict[str, Any]]):
+    if not f:
+        return None
+    kind = f.get("kind", "dense")
+    if kind == "dense":
+        return DenseFFNSpec(ff=int(f["ff"]), act="polynorm")
+    if kind != "moe":
+        raise ValueError(f"unknown feed-forward kind {kind!r}")
+    r = f["router"]
+    g = r.get("groups") or {}
+    E, n_g = int(r["experts"]), int(g.get("count", 1))
+    keep = int(g.get("keep", n_g))
+    if E % n_g or not 1 <= keep <= n_g:
+        raise ValueError("router: experts must split into equal groups")
+    if int(r["top"]) > keep * (E // n_g):
+        raise ValueError("router: top exceeds the experts of the kept groups")
+    return MoEFFNSpec(n_experts=E, top_k=int(r["top"]),
+                      ff=int(f["expert"]["ff"]), act="silu_glu",
+                      score="softmax_all", n_groups=n_g, keep_groups=keep)
+
+
+def looped_layer_specs_from_cfg(layers: List[Dict[str, Any]],
+                                loop: Optional[Dict[str, Any]]
+                                ) -> List[LayerSpec]:
+    """Pimodra: the list of layer RUNS in execution order. Layers
+    start..stop-1 of the checkpoint run `times` times in a row; every run
+    is a LayerSpec of its own (own pages), runs after the first pass name
+    the first pass's run as `weights_of`, and the first run of each pass
+    carries the pass number as `step_row`."""
+    n = len(layers)
+    order: List[Tuple[int, Optional[int]]] = [(i, None) for i in range(n)]
+    if loop:
+        a, b, times = int(loop["start"]), int(loop["stop"]), int(loop["times"])
+        if not (0 <= a < b <= n and times >= 1):
+            raise ValueError("loop: need 0 <= start < stop <= layers, times >= 1")
+        order = [(i, None) for i in range(a)]
+        for t in range(times):
+            order += [(i, t) for i in range(a, b)]
+        order += [(i, None) for i in range(b, n)]
+    out: List[LayerSpec] = []
+    first_run: Dict[int, int] = {}
+    for run, (i, t) in enumerate(order):
+        l = layers[i]
+        if l["type"] != "attention":
+            raise ValueError(f"unknown mixer type {l['type']!r}")
+        owner = first_run.setdefault(i, run)
+        out.append(LayerSpec(
+            mixer=_talk_attn_from_cfg(l["mixer"]),
+            ffn=_pimodra_ffn_from_cfg(l.get("mlp")), form="sandwich_w",
+            weights_of=None if owner == run else owner,
+            step_row=t if (t is not None and i == int(loop["start"])) else None,
+            src=i))
+    return out
+
+
 def complete_from_shapes(layers: List[LayerSpec],
                          shapes: Dict[str, Tuple[int, ...]]) -> None:
     """Sizes that only tensor shapes give: the low-rank widths of a delta
@@ -393,6 +533,10 @@ def hybrid_n_params(width: int, vocab: int, taps: int,
             if l.weights_of is None or active_only:
                 n += width + _parallel_layer_params(width, l)
             continue
+        if l.form == "sandwich_w":
+            if l.weights_of is None or active_only:
+                n += _sandwich_w_layer_params(width, l, active_only)
+            continue
         n += 4 + width * taps
         if m.kind == "latent_attention":
             n += width * (m.q_size + m.cache_dim + m.heads) + m.kv_rank
@@ -404,6 +548,19 @@ def hybrid_n_params(width: int, vocab: int, taps: int,
         if f is not None:
             e = f.top_k if active_only else f.n_experts
             n += width * f.n_experts + 3 * width * (e * f.ff + f.shared_ff)
+    return n
+
+
+def _sandwich_w_layer_params(width: int, l: LayerSpec,
+                             active_only: bool) -> int:
+    m, f = l.mixer, l.ffn
+    n = 2 * width + width * sum(sz for _, sz in m.in_sizes)
+    n += m.heads * m.heads + m.out_size * width
+    if isinstance(f, DenseFFNSpec):
+        n += 2 * width + 2 * width * f.ff + 4
+    elif f is not None:
+        e = f.top_k if active_only else f.n_experts
+        n += 2 * width + width * f.n_experts + 3 * width * e * f.ff
     return n
 
 
@@ -487,3 +644,33 @@ def nukopel_layers(n_layers: int, width: int, *, attn_every: int = 4,
             n_experts=experts, top_k=top_k, ff=ff, limit=limit,
             shared_ff=shared_ff, shared_limit=limit)))
     return out
+
+
+def pimodra_layers(n_layers: int, width: int, *, heads: int = 16,
+                   kv_heads: int = 2, dim: int = 128, window: int = 1024,
+                   ff: int = 8192, experts: int = 8, top_k: int = 2,
+                   expert_ff: int = 1024, groups: int = 4, keep: int = 2,
+                   moe_from: int = 1, loop: Optional[Tuple[int, int, int]] = None
+                   ) -> List[LayerSpec]:
+    """A synthetic Pimodra stack for benchmarks: head-mixing windowed
+    attention everywhere, a dense PolyNorm feed-forward in the layers
+    before `moe_from` and group-limited routed experts after; loop =
+    (start, stop, times) repeats a block with shared tensors."""
+    cfg_layers = []
+    for i in range(n_layers):
+        mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim,
+                 "scale": dim ** -0.5, "mask": {"size": window},
+                 "rot": {"base": 1e6, "dims": dim,
+                         "scaling": {"factor": 8.0, "original": 4096,
+                                     "fast": 32.0, "slow": 1.0}}}
+        if i < moe_from:
+            mlp: Dict[str, Any] = {"kind": "dense", "ff": ff}
+        else:
+            mlp = {"kind": "moe", "expert": {"ff": expert_ff},
+                   "router": {"experts": experts, "top": top_k,
+                              "groups": {"count": groups, "keep": keep}}}
+        cfg_layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+    lp = None
+    if loop:
+        lp = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return looped_layer_specs_from_cfg(cfg_layers, lp)

@@ -48,12 +48,17 @@ class ModelSpec:
     # vocab specials (byte-tokenizer defaults; overridden by a real tokenizer)
     bos_token_id: int = 1
     eos_token_id: int = 2
-    # hybrid stacks (arch "nukopel", "pugozen"): per-layer mixer/feed-forward specs
+    # hybrid stacks (arch "nukopel", "pugozen", "pimodra"): per-layer mixer/feed-forward specs
     # (models/hybrid.py). When set, the uniform-layer fields above hold
     # representative maxima only; the Runner's hybrid path reads these.
     layer_specs: Optional[List[Any]] = None
     embed_scale: float = 1.0     # x = embed[token] * embed_scale
     canon_taps: int = 0          # causal per-channel conv on the mixer input
+    norm_groups: int = 1         # weighted RMS norms over equal parts of a row
+    step_rows: int = 0           # rows of the per-pass residual step table
+    # the config.json "layers" / "loop" entries a looped stack was unrolled
+    # from (kept for export)
+    source_cfg: Optional[Dict[str, Any]] = None
 
     @property
     def is_hybrid(self) -> bool:
@@ -470,6 +475,31 @@ def pugozen_spec(name: str, cfg: Dict[str, Any],
     )
 
 
+def pimodra_spec(name: str, cfg: Dict[str, Any]) -> ModelSpec:
+    """Parse a Pimodra config.json dict: head-mixing windowed attention,
+    dense PolyNorm or group-routed expert feed-forwards, weighted grouped
+    norms around every sublayer, an optional repeated block of layers
+    (unrolled here into one layer spec per run), tied output embedding."""
+    from .hybrid import looped_layer_specs_from_cfg
+
+    loop = cfg.get("loop") or None
+    layers = looped_layer_specs_from_cfg(cfg["layers"], loop)
+    spec = hybrid_spec(
+        name, int(cfg["vocab"]), int(cfg["width"]), layers,
+        eps=float(cfg["norm"]["eps"]), embed_scale=1.0, canon_taps=0,
+        max_seq_len=int(cfg.get("max_seq_len", 32768)),
+        arch="pimodra", norm_type="group_rmsnorm", act_type="polynorm",
+    )
+    spec.tie_embeddings = True
+    spec.norm_groups = int(cfg["norm"].get("groups", 1))
+    if spec.hidden_size % spec.norm_groups:
+        raise ValueError("norm.groups must divide the width")
+    spec.step_rows = int(loop["times"]) if loop else 0
+    spec.n_kv_heads = max(l.mixer.kv_heads for l in layers)
+    spec.source_cfg = {"layers": cfg["layers"], "loop": loop}
+    return spec
+
+
 def resolve_spec(name: str, model_path: Optional[str] = None) -> ModelSpec:
     """Resolve a model name (preset / alias / HF id / local dir) to a spec.
 
@@ -514,6 +544,9 @@ def spec_from_hf_config(model_path: str, name: Optional[str] = None) -> ModelSpe
         return pugozen_spec(
             name or os.path.basename(os.path.normpath(model_path)), cfg,
             safetensors_shapes(model_path))
+    if cfg.get("architecture") == "Pimodra":
+        return pimodra_spec(
+            name or os.path.basename(os.path.normpath(model_path)), cfg)
     if cfg.get("model_type") == "gpt2" or "n_embd" in cfg:
         spec = _gpt2(
             name or cfg.get("_name_or_path", os.path.basename(model_path)),

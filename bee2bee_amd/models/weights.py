@@ -43,6 +43,9 @@ class LayerWeights:
         # projections incl. the feed-forward's up; mixer outputs + down),
         # their column layouts, and the mixer parts' small fp32 tensors
         "norm_w", "w_in", "w_out", "layout", "mix",
+        # weighted-sandwich layers: the four grouped-norm weights, the
+        # attention's head-mixing matrix, the dense activation's numbers
+        "norms", "talk", "act_coef",
     )
 
     def __init__(self) -> None:
@@ -73,6 +76,9 @@ class LayerWeights:
         self.w_out = None      # [width, out_total]
         self.layout = None     # models/hybrid.py fused_layout(layer)
         self.mix = None        # {part prefix: SimpleNamespace of tensors}
+        self.norms = None      # 4 x [width] fp32: pre/post mixer, pre/post ffn
+        self.talk = None       # [heads, heads] fp32
+        self.act_coef = None   # [4] fp32 (PolyNorm a, b, c, e)
 
 
 class ModelWeights:
@@ -86,6 +92,7 @@ class ModelWeights:
         self.final_norm_bias: Optional[torch.Tensor] = None
         self.lm_head: Optional[torch.Tensor] = None  # [vocab, hidden]
         self.final_gain: Optional[float] = None  # scalar-gain final norm
+        self.step_table: Optional[torch.Tensor] = None  # [passes, hidden] fp32
         self.layers = [LayerWeights() for _ in range(spec.n_layers)]
         # expert-parallel shard: when set, MoE expert tensors hold only
         # experts [lo, hi) (gate stays replicated); see parallel/ep.py
@@ -115,6 +122,8 @@ class ModelWeights:
                     "hybrid stacks are not sharded (pipeline/expert ranges)")
             if s.arch == "pugozen":
                 return self._random_init_pugozen(seed)
+            if s.arch == "pimodra":
+                return self._random_init_pimodra(seed)
             return self._random_init_hybrid(seed)
         lo, hi = layer_range or (0, s.n_layers)
         self.expert_range = expert_range
@@ -214,6 +223,8 @@ class ModelWeights:
                     "hybrid stacks are not sharded (pipeline/expert ranges)")
             if s.arch == "pugozen":
                 return self._load_pugozen(model_path)
+            if s.arch == "pimodra":
+                return self._load_pimodra(model_path)
             return self._load_nukopel(model_path)
         if s.arch == "gpt2":
             return self._load_gpt2(model_path, layer_range)
@@ -547,6 +558,128 @@ class ModelWeights:
                 lw.w_down = act(get(p + "mlp.shared.down"))
 
 
+
+    # ------------------------------------- weighted-sandwich (looped) stacks
+
+    @torch.no_grad()
+    def _load_pimodra(self, model_path: str) -> "ModelWeights":
+        """Pimodra safetensors: 'embed' (also the output matrix),
+        'final.norm', 'loop.step' [passes, width] when a block repeats, and
+        per checkpoint layer 'l<i>.norm1|norm1b|norm2|norm2b' [width],
+        'l<i>.mix.q|k|v|g|o|talk', 'l<i>.mlp.up|down|act' (dense) or
+        'l<i>.mlp.router|e<k>.gate|up|down' (experts). Linear weights
+        [out, in]."""
+        tensors = dict(iter_safetensors(model_path))
+        self._assemble_pimodra(lambda name: tensors.pop(name))
+        return self
+
+    @torch.no_grad()
+    def _random_init_pimodra(self, seed: int) -> "ModelWeights":
+        import zlib
+
+        def get(name: str) -> torch.Tensor:
+            tseed = (seed * 1000003 + zlib.crc32(name.encode())) % (2**31)
+            gen = torch.Generator(device=self.device).manual_seed(tseed)
+            shape, mean, std = self._pimodra_shape(name)
+            t = torch.randn(tuple(shape), generator=gen, dtype=torch.float32,
+                            device=self.device)
+            if name.endswith("mix.talk"):
+                # near the identity: a head keeps most of its own weights
+                t = torch.eye(shape[0], device=self.device) / std + t
+            return (mean + std * t).bfloat16()
+
+        self._assemble_pimodra(get)
+        return self
+
+    def _pimodra_shape(self, name: str):
+        """(shape, init mean, init std) of a checkpoint tensor."""
+        s = self.spec
+        W, V = s.hidden_size, s.vocab_size
+        if name == "embed":
+            return (V, W), 0.0, 1.0
+        if name == "final.norm":
+            return (W,), 1.0, 0.1
+        if name == "loop.step":
+            return (s.step_rows, W), 0.0, 0.5
+        head, rest = name.split(".", 1)
+        l = next(x for x in s.layer_specs if x.src == int(head[1:]))
+        m, f = l.mixer, l.ffn
+        lin = W ** -0.5
+        if rest in ("norm1", "norm1b", "norm2", "norm2b"):
+            return (W,), 1.0, 0.1
+        sizes = dict(m.in_sizes)
+        if rest in ("mix.q", "mix.k", "mix.v", "mix.g"):
+            return (sizes[rest[4:]], W), 0.0, lin
+        if rest == "mix.o":
+            return (W, m.out_size), 0.0, m.out_size ** -0.5
+        if rest == "mix.talk":
+            return (m.heads, m.heads), 0.0, 0.1
+        if rest == "mlp.up":
+            return (f.ff, W), 0.0, lin
+        if rest == "mlp.down":
+            return (W, f.ff), 0.0, f.ff ** -0.5
+        if rest == "mlp.act":
+            return (4,), 0.3, 0.2
+        if rest == "mlp.router":
+            return (f.n_experts, W), 0.0, lin
+        if rest.endswith(".down"):
+            return (W, f.ff), 0.0, f.ff ** -0.5
+        return (f.ff, W), 0.0, lin
+
+    def _assemble_pimodra(self, get) -> None:
+        """Engine layout of a weighted-sandwich stack: one fused input
+        projection per attention [q | k | v | gate], the head-mixing matrix
+        and all norm weights in fp32, the dense feed-forward's up matrix in
+        the single-fc slot, stacked expert matrices [E, 2ff, W] / [E, W, ff].
+        A run with weights_of shares the owning run's LayerWeights."""
+        s = self.spec
+        dev, dt = self.device, self.dtype
+
+        def act(t: torch.Tensor) -> torch.Tensor:
+            return t.to(dev, dt).contiguous()
+
+        def f32(t: torch.Tensor) -> torch.Tensor:
+            return t.to(dev, torch.float32).contiguous()
+
+        self.embed = act(get("embed"))
+        self.lm_head = self.embed
+        self.final_norm = f32(get("final.norm"))
+        if s.step_rows:
+            self.step_table = f32(get("loop.step"))
+        for i, l in enumerate(s.layer_specs):
+            if l.weights_of is not None:
+                continue
+            lw, p, m, f = self.layers[i], f"l{l.src}.", l.mixer, l.ffn
+            norms = []
+            for n_ in ("norm1", "norm1b", "norm2", "norm2b"):
+                if f is None and n_ in ("norm2", "norm2b"):
+                    norms.append(None)
+                else:
+                    norms.append(f32(get(p + n_)))
+            lw.norms = tuple(norms)
+            lw.wqkv = act(torch.cat([get(p + "mix.q"), get(p + "mix.k"),
+                                     get(p + "mix.v"), get(p + "mix.g")],
+                                    dim=0))
+            lw.talk = f32(get(p + "mix.talk"))
+            lw.wo = act(get(p + "mix.o"))
+            if f is None:
+                continue
+            if getattr(f, "n_experts", 0):
+                lw.moe_gate = f32(get(p + "mlp.router"))
+                lw.moe_w_gate_up = act(torch.stack([
+                    torch.cat([get(f"{p}mlp.e{e}.gate"),
+                               get(f"{p}mlp.e{e}.up")], dim=0)
+                    for e in range(f.n_experts)]))
+                lw.moe_w_down = act(torch.stack([
+                    get(f"{p}mlp.e{e}.down") for e in range(f.n_experts)]))
+            else:
+                lw.w_gate_up = act(get(p + "mlp.up"))
+                lw.w_down = act(get(p + "mlp.down"))
+                lw.act_coef = f32(get(p + "mlp.act"))
+        for i, l in enumerate(s.layer_specs):
+            if l.weights_of is not None:
+                self.layers[i] = self.layers[l.weights_of]
+
     # ------------------------------------------- parallel-form hybrid stacks
 
     @torch.no_grad()
@@ -723,6 +856,85 @@ class ModelWeights:
         for i, l in enumerate(s.layer_specs):
             if l.weights_of is not None:
                 self.layers[i] = self.layers[l.weights_of]
+
+
+def pimodra_config(spec: ModelSpec) -> Dict:
+    """The config.json dict of a Pimodra spec (inverse of pimodra_spec)."""
+    def mixer(m):
+        rot = {"base": m.rope_base, "dims": m.rope_dims}
+        if m.rope_scaling:
+            rot["scaling"] = dict(m.rope_scaling)
+        out = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim,
+               "vdim": m.vdim, "scale": m.scale, "rot": rot}
+        if m.window:
+            out["mask"] = {"size": m.window}
+        return out
+
+    def mlp(f):
+        if f is None:
+            return None
+        if getattr(f, "n_experts", 0):
+            return {"kind": "moe", "expert": {"ff": f.ff},
+                    "router": {"experts": f.n_experts, "top": f.top_k,
+                               "groups": {"count": f.n_groups,
+                                          "keep": f.keep_groups}}}
+        return {"kind": "dense", "ff": f.ff}
+
+    by_src = {}
+    for l in spec.layer_specs:
+        by_src.setdefault(l.src, l)
+    layers = [{"type": "attention", "mixer": mixer(by_src[i].mixer),
+               "mlp": mlp(by_src[i].ffn)} for i in sorted(by_src)]
+    cfg = {"architecture": "Pimodra", "vocab": spec.vocab_size,
+           "width": spec.hidden_size, "max_seq_len": spec.max_seq_len,
+           "norm": {"eps": spec.rms_eps, "groups": spec.norm_groups},
+           "layers": layers}
+    loop = (spec.source_cfg or {}).get("loop")
+    if loop:
+        cfg["loop"] = dict(loop)
+    return cfg
+
+
+def _save_pimodra(weights: "ModelWeights", out_dir: str, tensors, cpu) -> None:
+    from safetensors.torch import save_file
+
+    s = weights.spec
+
+    def put(name: str, t: torch.Tensor) -> None:
+        tensors[name] = cpu(t).to(torch.bfloat16)
+
+    put("embed", weights.embed)
+    put("final.norm", weights.final_norm)
+    if weights.step_table is not None:
+        put("loop.step", weights.step_table)
+    for i, l in enumerate(s.layer_specs):
+        if l.weights_of is not None:
+            continue
+        lw, p, m, f = weights.layers[i], f"l{l.src}.", l.mixer, l.ffn
+        for n_, t in zip(("norm1", "norm1b", "norm2", "norm2b"), lw.norms):
+            if t is not None:
+                put(p + n_, t)
+        off = 0
+        for n_, sz in m.in_sizes:
+            put(p + "mix." + n_, lw.wqkv[off : off + sz])
+            off += sz
+        put(p + "mix.talk", lw.talk)
+        put(p + "mix.o", lw.wo)
+        if f is None:
+            continue
+        if getattr(f, "n_experts", 0):
+            put(p + "mlp.router", lw.moe_gate)
+            for e in range(f.n_experts):
+                put(f"{p}mlp.e{e}.gate", lw.moe_w_gate_up[e, : f.ff])
+                put(f"{p}mlp.e{e}.up", lw.moe_w_gate_up[e, f.ff :])
+                put(f"{p}mlp.e{e}.down", lw.moe_w_down[e])
+        else:
+            put(p + "mlp.up", lw.w_gate_up)
+            put(p + "mlp.down", lw.w_down)
+            put(p + "mlp.act", lw.act_coef)
+    save_file(tensors, os.path.join(out_dir, "model.safetensors"))
+    with open(os.path.join(out_dir, "config.json"), "w") as fh:
+        json.dump(pimodra_config(s), fh, indent=1)
 
 
 def safetensors_shapes(model_path: str) -> Dict[str, Tuple[int, ...]]:
@@ -1016,6 +1228,8 @@ def save_hf(weights: ModelWeights, out_dir: str) -> None:
     if s.is_hybrid:
         if s.arch == "pugozen":
             _save_pugozen(weights, out_dir, tensors, cpu)
+        elif s.arch == "pimodra":
+            _save_pimodra(weights, out_dir, tensors, cpu)
         else:
             _save_nukopel(weights, out_dir, tensors, cpu)
         return

@@ -416,3 +416,64 @@ def retention_attn(q, k, v, decay, rope_dims: int, cos, sin, k_scale: float,
     return reference.retention_attn(q, k, v, decay, rope_dims, cos, sin,
                                     k_scale, state, state_slots, cu_seqlens,
                                     positions)
+
+
+# ----------------------------------------------- weighted-sandwich stacks
+# (ops/reference.py documents shapes and formulas)
+
+rope_tables_scaled = reference.rope_tables_scaled
+
+
+def add_group_rmsnorm(resid, y, w_post, step, w_pre, groups: int, eps: float,
+                      out_dtype):
+    """resid(fp32) += group_norm(y) * w_post [+ step] in place; ->
+    group_norm(resid) * w_pre (None when w_pre is None). y None: only the
+    step and the norm. One pass over HBM per operand on the GPU."""
+    if _use_hip(resid):
+        return require_hip().add_group_rmsnorm(resid, y, w_post, step, w_pre,
+                                               groups, eps, out_dtype)
+    return reference.add_group_rmsnorm(resid, y, w_post, step, w_pre, groups,
+                                       eps, out_dtype)
+
+
+def rope_unit_store(q, k, v, eps: float, rope_dims: int, positions, cos, sin,
+                    q_mult: float, k_cache, v_cache, slot_mapping) -> None:
+    if _use_hip(q):
+        require_hip().rope_unit_store(q, k, v, eps, rope_dims, positions, cos,
+                                      sin, float(q_mult), k_cache, v_cache,
+                                      slot_mapping)
+        return
+    reference.rope_unit_store(q, k, v, eps, rope_dims, positions, cos, sin,
+                              q_mult, k_cache, v_cache, slot_mapping)
+
+
+def talk_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
+              cu_seqlens, talk, gate, window: int, out,
+              max_qlen: int = 0) -> None:
+    """max_qlen: longest chunk of the step (host int); with bf16 pages, a
+    matrix-core head size and a chunk of at least 16 rows the step takes
+    the query-tiled kernel."""
+    if _use_hip(q):
+        require_hip().talk_attn(q, k_cache, v_cache, block_table, positions,
+                                seq_idx, cu_seqlens, talk, gate, window, out,
+                                max_qlen)
+        return
+    reference.talk_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
+                        cu_seqlens, talk, gate, window, out)
+
+
+def polynorm(z, coef, eps: float, out_dtype):
+    if _use_hip(z):
+        return require_hip().polynorm(z, coef, eps, out_dtype)
+    return reference.polynorm(z, coef, eps, out_dtype)
+
+
+def silu_glu(gate_up):
+    if _use_hip(gate_up):
+        return require_hip().silu_glu(gate_up)
+    return reference.silu_glu(gate_up)
+
+
+def group_topk_gate(logits, top_k: int, n_groups: int, keep_groups: int):
+    # [T, E] gating math: torch ops on both devices, like moe_topk_gate
+    return reference.group_topk_gate(logits, top_k, n_groups, keep_groups)

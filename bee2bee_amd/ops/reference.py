@@ -18,6 +18,7 @@ RoPE is llama-style rotate_half: pair (i, i + hd/2).
 """
 from __future__ import annotations
 
+import math
 from typing import Optional, Tuple
 
 import torch
@@ -815,3 +816,187 @@ def retention_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                 (kc * tail[..., None]).transpose(1, 2), vc)
         state[slot] = S
     return out.view(T, H * Dv)
+
+
+# --------------------------------------------- weighted-sandwich stacks
+#
+# Mechanisms of stacks whose sublayers are x += norm_b(f(norm_a(x))) with
+# weighted RMS norms over equal parts of a row: the grouped norm fused with
+# the fp32 residual update, rotation tables with wavelength-dependent
+# frequency scaling, "rotate, then unit-norm" query/key preparation with the
+# page store, windowed attention whose softmax weights are mixed across
+# heads, the PolyNorm activation, the plain gated-linear-unit, and
+# group-limited expert choice.
+
+
+def group_rmsnorm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """fp32 rows [T, W] -> each of `groups` equal consecutive parts divided
+    by its own sqrt(mean^2 + eps), the row times w; out_dtype."""
+    T, W = x.shape
+    xf = x.float().view(T, groups, W // groups)
+    r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return ((xf * r).view(T, W) * w.float()).to(out_dtype)
+
+
+def add_group_rmsnorm(resid: torch.Tensor, y: Optional[torch.Tensor],
+                      w_post: Optional[torch.Tensor],
+                      step: Optional[torch.Tensor],
+                      w_pre: Optional[torch.Tensor], groups: int, eps: float,
+                      out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """resid (fp32, in place) += group_norm(y) * w_post   (when y is given)
+    resid += step                                      (when step is given)
+    returns group_norm(resid) * w_pre                  (None if w_pre is)."""
+    if y is not None:
+        resid.add_(group_rmsnorm(y, w_post, groups, eps, torch.float32))
+    if step is not None:
+        resid.add_(step.float())
+    if w_pre is None:
+        return None
+    return group_rmsnorm(resid, w_pre, groups, eps, out_dtype)
+
+
+def rope_tables_scaled(max_len: int, dims: int, base: float,
+                       scaling: Optional[dict], device
+                       ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """cos/sin [max_len, dims/2], float64 angles rounded once to fp32.
+    Pair i turns at f_i = base^(-2i/dims). scaling {factor, original, fast,
+    slow}: with n(t) = dims ln(original / (2 pi t)) / (2 ln base), lo =
+    max(floor(n(fast)), 0), hi = min(ceil(n(slow)), dims - 1) and ramp_i =
+    clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the pair turns at
+    f_i / factor * ramp_i + f_i (1 - ramp_i), and cos and sin carry the
+    factor 0.1 ln(factor) + 1."""
+    half = dims // 2
+    i = torch.arange(half, dtype=torch.float64)
+    inv = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                    -2.0 * i / dims)
+    mag = 1.0
+    if scaling:
+        factor = float(scaling["factor"])
+
+        def n_of(turns: float) -> float:
+            return dims * math.log(float(scaling["original"]) /
+                                   (2.0 * math.pi * turns)) / (
+                                       2.0 * math.log(float(base)))
+
+        lo = max(math.floor(n_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(n_of(float(scaling["slow"]))), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        inv = inv / factor * ramp + inv * (1.0 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    ang = torch.outer(torch.arange(max_len, dtype=torch.float64), inv)
+    return ((ang.cos() * mag).to(device, torch.float32),
+            (ang.sin() * mag).to(device, torch.float32))
+
+
+def rope_unit_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                    eps: float, rope_dims: int, positions: torch.Tensor,
+                    cos, sin, q_mult: float, k_cache: torch.Tensor,
+                    v_cache: torch.Tensor,
+                    slot_mapping: torch.Tensor) -> None:
+    """q [T, H, D] (view, rewritten in place): unit(rotate(q)) * q_mult.
+    k [T, G, D], v [T, G, Dv] (views, left as they are): unit(rotate(k))
+    goes to k_cache [n_blocks, G, block, D], v to v_cache
+    [n_blocks, G, block, Dv], at slot_mapping. unit = x / sqrt(mean(x^2) +
+    eps) per head, no weight, AFTER the rotation."""
+    bs = k_cache.shape[2]
+    qf, kf = q.float(), k.float()
+    if rope_dims:
+        p = positions.long()
+        c, s = cos[p][:, None], sin[p][:, None]
+        qf = _rot_half(qf, c, s, rope_dims)
+        kf = _rot_half(kf, c, s, rope_dims)
+    qf = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * q_mult
+    kf = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps)
+    q.copy_(qf.to(q.dtype))
+    slot = slot_mapping.long()
+    blk, off = slot // bs, slot % bs
+    k_cache[blk, :, off] = kf.to(k_cache.dtype)
+    v_cache[blk, :, off] = v.to(v_cache.dtype)
+
+
+def talk_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+              block_table: torch.Tensor, positions: torch.Tensor,
+              seq_idx: torch.Tensor, cu_seqlens: torch.Tensor,
+              talk: torch.Tensor, gate: torch.Tensor, window: int,
+              out: torch.Tensor) -> None:
+    """Grouped-query attention over the pages whose softmax weights are
+    mixed across heads: scores q . k (every multiplier is already in q), row
+    t at position p of chunk b sees cached positions j <= p (j > p - window
+    when window > 0), w_g = softmax per head, w'_h = sum_g talk[h, g] w_g,
+    o_h = w'_h applied to the values of head h's own key/value head.
+    out [T, H * Dv] (strided view) <- o * sigmoid(gate) (gate raw,
+    [T, H * Dv], strided view)."""
+    T, H, D = q.shape
+    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    rep = H // G
+    cu = cu_seqlens.tolist()
+    res = torch.zeros(T, H, Dv, dtype=torch.float32, device=q.device)
+    tk = talk.float()
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        pos = positions[lo:hi].long()
+        k_lo = max(0, int(pos.min()) - window + 1) if window > 0 else 0
+        k_hi = int(pos.max()) + 1
+        kpos = torch.arange(k_lo, k_hi, device=q.device)
+        blk = block_table[b].long()[kpos // bs]
+        keys = k_cache[blk, :, kpos % bs].float()          # [S, G, D]
+        vals = v_cache[blk, :, kpos % bs].float()          # [S, G, Dv]
+        qb = q[lo:hi].float().view(hi - lo, G, rep, D)
+        s = torch.einsum("tgrd,sgd->grts", qb, keys)
+        d = pos[:, None] - kpos[None, :]
+        dead = d < 0
+        if window > 0:
+            dead = dead | (d >= window)
+        s.masked_fill_(dead[None, None], float("-inf"))
+        w = torch.softmax(s, dim=-1).reshape(H, hi - lo, -1)   # [H, t, S]
+        w = torch.einsum("hg,gts->hts", tk, w).view(G, rep, hi - lo, -1)
+        o = torch.einsum("grts,sgv->tgrv", w, vals)
+        res[lo:hi] = o.reshape(hi - lo, H, Dv)
+    g = torch.sigmoid(gate.float())
+    out.copy_((res.view(T, H * Dv) * g).to(out.dtype))
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float,
+             out_dtype: torch.dtype) -> torch.Tensor:
+    """[T, N] -> a unit(z) + b unit(z^2) + c unit(z^3) + e, (a, b, c, e) =
+    coef, powers element by element, unit over the row; fp32 inside."""
+    zf = z.float()
+    c = coef.float()
+
+    def unit(x):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+    z2 = zf * zf
+    y = c[0] * unit(zf) + c[1] * unit(z2) + c[2] * unit(z2 * zf) + c[3]
+    return y.to(out_dtype)
+
+
+def silu_glu(gate_up: torch.Tensor) -> torch.Tensor:
+    """[..., 2I] -> [..., I]: silu(gate) * up."""
+    g, u = gate_up.float().chunk(2, dim=-1)
+    return (torch.nn.functional.silu(g) * u).to(gate_up.dtype)
+
+
+def group_topk_gate(logits: torch.Tensor, top_k: int, n_groups: int,
+                    keep_groups: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Group-limited choice on softmax scores. logits fp32 [T, E]: scores =
+    softmax over all experts; experts form n_groups equal groups of
+    neighbours, a group's score is its largest expert score, experts outside
+    the best keep_groups groups cannot be chosen; the top_k remaining scores
+    are the weights, as they are. -> (weights [T, k] fp32, idx [T, k] int32).
+    Fixed shapes and no host sync (graph-capturable)."""
+    T, E = logits.shape
+    s = torch.softmax(logits.float(), dim=-1)
+    pick = s
+    if n_groups > 1 and keep_groups < n_groups:
+        gs = s.view(T, n_groups, E // n_groups).max(-1).values
+        top_g = torch.topk(gs, keep_groups, dim=-1).indices
+        allow = torch.zeros(T, n_groups, dtype=torch.bool, device=s.device)
+        allow.scatter_(1, top_g, True)
+        allow = allow[:, :, None].expand(T, n_groups, E // n_groups)
+        pick = torch.where(allow.reshape(T, E), s, torch.full_like(s, -1.0))
+    idx = torch.topk(pick, top_k, dim=-1).indices
+    return s.gather(1, idx), idx.to(torch.int32)
