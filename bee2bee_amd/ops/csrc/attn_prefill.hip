@@ -485,3 +485,266 @@ extern "C" int launch_attn_prefill_paged_sink(
             s_o);
     return 0;
 }
+
+// ---------------------------------------------------------- cross-value mfma
+// The paged MFMA prefill kernel for attention whose softmax weights are
+// mixed across heads afterwards: every query head's weights (bf16 hi+lo
+// pair) are applied to the values of ALL key/value heads, so the mix can
+// be taken on the per-(query head, value head) sums:
+//   part[t, h, n, :] = sum_j softmax_h(j) v_n(j)      (normalized, fp32).
+// Scores use head h's own key head. window > 0: row at absolute position p
+// sees keys p - window < j <= p; key tiles wholly before the tile's first
+// window are skipped. Same tiling and fragment maps as attn_prefill_mfma;
+// the V^T tile is staged once per value head against the same P tile.
+template <int HD, int NV>
+__global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
+    const unsigned short* __restrict__ q,
+    const unsigned short* __restrict__ k,  // k_cache [nb,nkv,bs,HD]
+    const unsigned short* __restrict__ v,  // v_cache [nb,nkv,bs,HD]
+    const int* __restrict__ cu, const int* __restrict__ block_table,
+    const int* __restrict__ seq_lens, float* __restrict__ part, int nq,
+    int nkv, long s_q, int W, int bs, int window) {
+    constexpr int KSTEPS = HD / 32;
+    const int seq = blockIdx.z;
+    const int h = blockIdx.y;
+    const int kvh = h / (nq / nkv);
+    const int s0 = cu[seq], s1 = cu[seq + 1];
+    const int QL = s1 - s0;
+    const int L = seq_lens[seq];
+    const int hist = L - QL;
+    const int* bt = block_table + (long)seq * W;
+    const int q0 = blockIdx.x * PF_TM;
+    if (q0 >= QL) return;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % WAVE;
+    const int wid = tid / WAVE;
+    const int lg = lane >> 4;
+    const int li = lane & 15;
+
+    extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+    constexpr int VT_STRIDE = PF_TN + PF_PAD;
+    constexpr int K_ELEMS = PF_TN * (HD + PF_PAD);
+    constexpr int P_TILE = PF_TM * VT_STRIDE;
+    constexpr int P_ELEMS = P_TILE * 2;
+    constexpr int VT_OFF = (K_ELEMS > P_ELEMS ? K_ELEMS : P_ELEMS);
+    unsigned short* k_s = reinterpret_cast<unsigned short*>(smem_raw);
+    unsigned short* vt_s = k_s + VT_OFF;
+
+    bf16x8 a_q[KSTEPS];
+    const int my_qrow = q0 + wid * PF_QROWS + li;
+    const bool row_ok = my_qrow < QL;
+    {
+        const unsigned short* qr = q + (long)(s0 + my_qrow) * s_q + (long)h * HD;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            const int d = ks * 32 + lg * 8;
+            if (row_ok) {
+                a_q[ks] = *reinterpret_cast<const bf16x8*>(qr + d);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a_q[ks][e] = (__bf16)0.f;
+            }
+        }
+    }
+
+    float m_run[4], l_run[4];
+    f32x4 o_acc[NV][HD / 16];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { m_run[r] = -1e30f; l_run[r] = 0.f; }
+#pragma unroll
+    for (int n = 0; n < NV; ++n)
+#pragma unroll
+        for (int nb = 0; nb < HD / 16; ++nb)
+            o_acc[n][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int kv_end = min(L, hist + q0 + PF_TM);
+    int kb0 = 0;
+    if (window > 0) kb0 = max(0, hist + q0 - window + 1) / PF_TN * PF_TN;
+    constexpr int THREADS_PER_ROW = HD / 8;
+
+    for (int kb = kb0; kb < kv_end; kb += PF_TN) {
+        // ---- stage K tile [64][HD] (own key head) and V^T of value head 0
+        __syncthreads();
+        for (int i = tid; i < PF_TN * THREADS_PER_ROW; i += 256) {
+            const int key = i / THREADS_PER_ROW;
+            const int d = (i % THREADS_PER_ROW) * 8;
+            const int gk = kb + key;
+            bf16x8 kraw{}, vraw{};
+            if (gk < kv_end) {
+                const long base = (long)bt[gk / bs] * nkv * bs + gk % bs;
+                kraw = load_kv8_bf16(k + (base + (long)kvh * bs) * HD + d);
+                vraw = load_kv8_bf16(v + base * HD + d);
+            }
+            *reinterpret_cast<bf16x8*>(k_s + key * (HD + PF_PAD) + d) = kraw;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                vt_s[(d + e) * VT_STRIDE + key] =
+                    ((const unsigned short*)&vraw)[e];
+        }
+        __syncthreads();
+
+        f32x4 sfrag[PF_TN / 16];
+#pragma unroll
+        for (int f = 0; f < PF_TN / 16; ++f) {
+            f32x4 acc{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                bf16x8 bk = *reinterpret_cast<const bf16x8*>(
+                    k_s + (f * 16 + li) * (HD + PF_PAD) + ks * 32 + lg * 8);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_q[ks], bk, acc,
+                                                              0, 0, 0);
+            }
+            sfrag[f] = acc;
+        }
+
+        float pmax[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pmax[r] = -1e30f;
+#pragma unroll
+        for (int f = 0; f < PF_TN / 16; ++f) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int qrow = q0 + wid * PF_QROWS + lg * 4 + r;
+                const int key = kb + f * 16 + li;
+                const int p = hist + qrow;
+                if (key > p || qrow >= QL || key >= kv_end ||
+                    (window > 0 && key <= p - window))
+                    sfrag[f][r] = -1e30f;
+                pmax[r] = fmaxf(pmax[r], sfrag[f][r]);
+            }
+        }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                pmax[r] = fmaxf(pmax[r], __shfl_xor(pmax[r], off));
+
+        float alpha[4], psum[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float mn = fmaxf(m_run[r], pmax[r]);
+            alpha[r] = __expf(m_run[r] - mn);
+            m_run[r] = mn;
+            psum[r] = 0.f;
+        }
+        unsigned short* p_s = k_s;  // the K tile becomes the P tiles (hi, lo)
+        __syncthreads();
+#pragma unroll
+        for (int f = 0; f < PF_TN / 16; ++f) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float pv = __expf(sfrag[f][r] - m_run[r]);
+                if (sfrag[f][r] <= -1e29f) pv = 0.f;
+                psum[r] += pv;
+                const int pi =
+                    (wid * PF_QROWS + lg * 4 + r) * VT_STRIDE + f * 16 + li;
+                const unsigned short hi = f2bf(pv);
+                p_s[pi] = hi;
+                p_s[P_TILE + pi] = f2bf(pv - bf2f(hi));
+            }
+        }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) psum[r] += __shfl_xor(psum[r], off);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            l_run[r] = l_run[r] * alpha[r] + psum[r];
+#pragma unroll
+        for (int n = 0; n < NV; ++n)
+#pragma unroll
+            for (int nb = 0; nb < HD / 16; ++nb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o_acc[n][nb][r] *= alpha[r];
+
+        __syncthreads();
+        bf16x8 a_p[PF_TN / 32], a_pl[PF_TN / 32];
+#pragma unroll
+        for (int ks2 = 0; ks2 < PF_TN / 32; ++ks2) {
+            const int pi = (wid * PF_QROWS + li) * VT_STRIDE + ks2 * 32 + lg * 8;
+            a_p[ks2] = *reinterpret_cast<const bf16x8*>(p_s + pi);
+            a_pl[ks2] = *reinterpret_cast<const bf16x8*>(p_s + P_TILE + pi);
+        }
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            if (n >= nkv) break;            // uniform over the workgroup
+            if (n > 0) {
+                // every wave is done with the previous value head's tile
+                __syncthreads();
+                for (int i = tid; i < PF_TN * THREADS_PER_ROW; i += 256) {
+                    const int key = i / THREADS_PER_ROW;
+                    const int d = (i % THREADS_PER_ROW) * 8;
+                    const int gk = kb + key;
+                    bf16x8 vraw{};
+                    if (gk < kv_end) {
+                        const long base =
+                            (long)bt[gk / bs] * nkv * bs + gk % bs;
+                        vraw = load_kv8_bf16(v + (base + (long)n * bs) * HD + d);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        vt_s[(d + e) * VT_STRIDE + key] =
+                            ((const unsigned short*)&vraw)[e];
+                }
+                __syncthreads();
+            }
+#pragma unroll
+            for (int nb = 0; nb < HD / 16; ++nb) {
+#pragma unroll
+                for (int ks2 = 0; ks2 < PF_TN / 32; ++ks2) {
+                    bf16x8 bv = *reinterpret_cast<const bf16x8*>(
+                        vt_s + (nb * 16 + li) * VT_STRIDE + ks2 * 32 + lg * 8);
+                    o_acc[n][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        a_p[ks2], bv, o_acc[n][nb], 0, 0, 0);
+                    o_acc[n][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        a_pl[ks2], bv, o_acc[n][nb], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    const int orow_base = q0 + wid * PF_QROWS;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int qrow = orow_base + lg * 4 + r;
+        if (qrow >= QL) continue;
+        const float inv = (l_run[r] > 0.f) ? 1.f / l_run[r] : 0.f;
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            if (n >= nkv) break;
+            float* orow = part + (((long)(s0 + qrow) * nq + h) * nkv + n) * HD;
+#pragma unroll
+            for (int nb = 0; nb < HD / 16; ++nb)
+                orow[nb * 16 + li] = o_acc[n][nb][r] * inv;
+        }
+    }
+}
+
+// Packed bf16 query chunks against the paged history, each query head's
+// softmax weights applied to every value head: part [T, nq, nkv, hd] fp32.
+// Head size 64 or 128 and nkv <= 4 (returns nonzero otherwise); every score
+// multiplier is already in q.
+extern "C" int launch_attn_prefill_paged_cross(
+    const unsigned short* q, long s_q, const unsigned short* k_cache,
+    const unsigned short* v_cache, const int* cu, const int* block_table,
+    const int* seq_lens, float* part, int nseq, int nq, int nkv, int hd,
+    int W, int bs, int max_qlen, int window, hipStream_t stream) {
+    if ((hd != 64 && hd != 128) || nkv > 4 || nkv < 1) return 1;
+    if (nseq == 0 || max_qlen == 0) return 0;
+    const int tiles = (max_qlen + PF_TM - 1) / PF_TM;
+    dim3 grid(tiles, nq, nseq);
+    const int smem = prefill_mfma_smem(hd, 1);
+#define PFC(HDV, NVV)                                                          \
+    hipLaunchKernelGGL((attn_prefill_cross_mfma<HDV, NVV>), grid, dim3(256),   \
+                       smem, stream, q, k_cache, v_cache, cu, block_table,     \
+                       seq_lens, part, nq, nkv, s_q, W, bs, window)
+    const int nv = nkv > 2 ? 4 : nkv;
+    if (hd == 128) {
+        if (nv == 4) PFC(128, 4); else if (nv == 2) PFC(128, 2); else PFC(128, 1);
+    } else {
+        if (nv == 4) PFC(64, 4); else if (nv == 2) PFC(64, 2); else PFC(64, 1);
+    }
+#undef PFC
+    return 0;
+}

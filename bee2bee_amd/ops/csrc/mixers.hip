@@ -1440,3 +1440,299 @@ extern "C" int launch_sink_attn(const void* q, long q_tok,
         seq_idx, sink, out, out_tok, out_scale, part_acc, part_ml, splits, Tn,
         H, G, D, Dv, bs, window, s);
 }
+
+// ---------------------------------------------------------------------------
+// talk_attn: windowed grouped-query softmax attention whose per-head softmax
+// weights are mixed across heads before they meet the values,
+//   w'_h = sum_g talk[h, g] w_g,   o_h = sum_j w'_h(j) v_{c(h)}(j),
+// c(h) the key/value head of query head h. Since the mix is linear,
+//   o_h = sum_g talk[h, g] A[g, c(h)],   A[g, c] = sum_j w_g(j) v_c(j):
+// every query head's ordinary softmax weights are applied to the values of
+// EVERY key/value head (kernel 1, online softmax, key-split capable), and a
+// second kernel merges the key splits, normalizes, mixes the heads with
+// `talk`, applies the sigmoid output gate and writes the activation.
+//
+// Kernel 1 keeps sink_attn's wave layout: one wave per (token, REP query
+// heads of one key group, block of NV value heads, key split); lane = key
+// for the scores, lane = coordinate pair for the value sums. Partials:
+// part_acc [S, T, H, G, Dv] (unnormalized), part_ml [S, T, H, 2].
+namespace {
+
+template <typename T, int DPL, int REP, int NV, bool PAIR>
+__global__ void __launch_bounds__(SA_WAVES * WAVE)
+talk_attn_kernel(const T* __restrict__ q, long q_tok,
+                 const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                 const int* __restrict__ block_table, int bt_stride,
+                 const int* __restrict__ positions,
+                 const int* __restrict__ seq_idx,
+                 float* __restrict__ part_acc, float* __restrict__ part_ml,
+                 int Tn, int H, int G, int D, int Dv, int bs, int window,
+                 int units, int vblocks) {
+    extern __shared__ __attribute__((aligned(16))) float sa_q[];
+    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int t = blockIdx.x;
+    const int u = blockIdx.y * SA_WAVES + wid;
+    if (u >= units * vblocks) return;      // no workgroup barrier below
+    const int h0 = (u % units) * REP;      // REP consecutive query heads
+    const int v0 = (u / units) * NV;       // NV consecutive value heads
+    const int split = blockIdx.z, nsplit = gridDim.z;
+    const int p = positions[t];
+    const int g = h0 / (H / G);
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int per =
+        ((p + 1 - lo + nsplit - 1) / nsplit + WAVE - 1) / WAVE * WAVE;
+    const int klo = lo + split * per, khi = min(p + 1, klo + per);
+    float* qv = sa_q + (long)wid * REP * D;
+    for (int i = lane; i < REP * D; i += WAVE)
+        qv[i] = ldf(q + (long)t * q_tok + (long)h0 * D + i);
+    WAVE_LDS_SYNC();
+    const int* bt = block_table + (long)seq_idx[t] * bt_stride;
+    float m[REP], l[REP], acc[NV][REP][DPL];
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+        m[r] = -INFINITY;
+        l[r] = 0.f;
+#pragma unroll
+        for (int n = 0; n < NV; ++n)
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) acc[n][r][i] = 0.f;
+    }
+    for (int j0 = klo; j0 < khi; j0 += WAVE) {
+        const int j = j0 + lane;
+        const bool valid = j < khi;
+        int row0 = 0;           // row of key head 0; lanes past the end
+        float sc[REP], pj[REP]; // point at a real row
+#pragma unroll
+        for (int r = 0; r < REP; ++r) sc[r] = 0.f;
+        const int nk = min(WAVE, khi - j0);
+        if (valid) row0 = bt[j / bs] * G * bs + j % bs;
+        if (valid)
+            SaDots<T, REP>::run(k_cache + (long)(row0 + g * bs) * D, qv, D,
+                                sc);
+#pragma unroll
+        for (int r = 0; r < REP; ++r) {
+            const float s = valid ? sc[r] : -INFINITY;
+            const float m_new = fmaxf(m[r], wave_max(s));
+            pj[r] = valid ? expf(s - m_new) : 0.f;
+            const float corr = expf(m[r] - m_new);
+            l[r] = l[r] * corr + wave_sum(pj[r]);
+#pragma unroll
+            for (int n = 0; n < NV; ++n)
+#pragma unroll
+                for (int i = 0; i < DPL; ++i) acc[n][r][i] *= corr;
+            m[r] = m_new;
+        }
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            if (v0 + n >= G) break;
+            for (int jj = 0; jj < nk; jj += SA_PV) {
+                float vv[SA_PV][DPL];
+#pragma unroll
+                for (int x = 0; x < SA_PV; ++x) {
+                    const T* vr =
+                        v_cache +
+                        (long)(__builtin_amdgcn_readlane(row0, jj + x) +
+                               (v0 + n) * bs) * Dv;
+                    if constexpr (PAIR) {
+#pragma unroll
+                        for (int i = 0; i < DPL; i += 2) {
+                            const int d = sa_coord<true>(lane, i);
+                            vv[x][i] = vv[x][i + 1] = 0.f;
+                            if (d < Dv) sa_ld2(vr + d, vv[x][i], vv[x][i + 1]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < DPL; ++i) {
+                            const int d = sa_coord<false>(lane, i);
+                            vv[x][i] = d < Dv ? ldf(vr + d) : 0.f;
+                        }
+                    }
+                }
+#pragma unroll
+                for (int x = 0; x < SA_PV; ++x)
+#pragma unroll
+                    for (int r = 0; r < REP; ++r) {
+                        const float pb = __builtin_bit_cast(
+                            float, __builtin_amdgcn_readlane(
+                                       __builtin_bit_cast(int, pj[r]), jj + x));
+#pragma unroll
+                        for (int i = 0; i < DPL; ++i)
+                            acc[n][r][i] += pb * vv[x][i];
+                    }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+        const int h = h0 + r;
+        const long prow = ((long)split * Tn + t) * H + h;
+        if (lane == 0 && v0 == 0) {
+            part_ml[prow * 2] = m[r];
+            part_ml[prow * 2 + 1] = l[r];
+        }
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            if (v0 + n >= G) break;
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) {
+                const int d = sa_coord<PAIR>(lane, i);
+                if (d < Dv)
+                    part_acc[(prow * G + v0 + n) * Dv + d] = acc[n][r][i];
+            }
+        }
+    }
+}
+
+// Merge of the key splits + head mix + output gate. Workgroup per token.
+// part_ml == nullptr: the partials are already normalized (one split).
+// LDS: wts [S*H] | talk [H*H] | A_c [H*Dv].
+template <typename T>
+__global__ void __launch_bounds__(256)
+talk_mix_kernel(const float* __restrict__ part_acc,
+                const float* __restrict__ part_ml,
+                const float* __restrict__ talk, const T* __restrict__ gate,
+                long gate_tok, T* __restrict__ out, long out_tok, int splits,
+                int Tn, int H, int G, int Dv) {
+    extern __shared__ __attribute__((aligned(16))) float tm_s[];
+    float* wts = tm_s;
+    float* tk = wts + splits * H;
+    float* A = tk + H * H;
+    const int t = blockIdx.x;
+    const int rep = H / G;
+    for (int h = threadIdx.x; h < H; h += blockDim.x) {
+        if (!part_ml) {
+            wts[h] = 1.f;
+            continue;
+        }
+        float M = -INFINITY;
+        for (int s = 0; s < splits; ++s) {
+            const long row = ((long)s * Tn + t) * H + h;
+            if (part_ml[row * 2 + 1] > 0.f) M = fmaxf(M, part_ml[row * 2]);
+        }
+        float L = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const long row = ((long)s * Tn + t) * H + h;
+            const float l = part_ml[row * 2 + 1];
+            const float w = l > 0.f ? expf(part_ml[row * 2] - M) : 0.f;
+            wts[s * H + h] = w;
+            L += l * w;
+        }
+        const float rcp = L > 0.f ? 1.f / L : 0.f;
+        for (int s = 0; s < splits; ++s) wts[s * H + h] *= rcp;
+    }
+    for (int i = threadIdx.x; i < H * H; i += blockDim.x) tk[i] = talk[i];
+    __syncthreads();
+    for (int c = 0; c < G; ++c) {
+        for (int idx = threadIdx.x; idx < H * Dv; idx += blockDim.x) {
+            const int gq = idx / Dv, d = idx - gq * Dv;
+            float a = 0.f;
+            for (int s = 0; s < splits; ++s)
+                a += wts[s * H + gq] *
+                     part_acc[((((long)s * Tn + t) * H + gq) * G + c) * Dv + d];
+            A[idx] = a;
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < rep * Dv; idx += blockDim.x) {
+            const int hl = idx / Dv, d = idx - hl * Dv;
+            const int h = c * rep + hl;
+            float o = 0.f;
+            for (int gq = 0; gq < H; ++gq) o += tk[h * H + gq] * A[gq * Dv + d];
+            const float gt =
+                ldf(gate + (long)t * gate_tok + (long)h * Dv + d);
+            stf(out + (long)t * out_tok + (long)h * Dv + d,
+                o / (1.f + expf(-gt)));
+        }
+        __syncthreads();
+    }
+}
+
+}  // namespace
+
+#define TA_LAUNCH(N, R, V, P)                                                 \
+    talk_attn_kernel<TT, N, R, V, P><<<grid, SA_WAVES * WAVE, smem, s>>>(     \
+        (const TT*)q, q_tok, (const TT*)k_cache, (const TT*)v_cache,          \
+        block_table, bt_stride, positions, seq_idx, part_acc, part_ml, Tn, H, \
+        G, D, Dv, bs, window, units, vblocks)
+
+#define TA_CASE(N, P)                                                         \
+    if (dpl == N && pair == P) {                                              \
+        if (rep == 4 && nv == 4) TA_LAUNCH(N, 4, 4, P);                       \
+        else if (rep == 4 && nv == 2) TA_LAUNCH(N, 4, 2, P);                  \
+        else if (rep == 4) TA_LAUNCH(N, 4, 1, P);                             \
+        else if (rep == 2 && nv == 4) TA_LAUNCH(N, 2, 4, P);                  \
+        else if (rep == 2 && nv == 2) TA_LAUNCH(N, 2, 2, P);                  \
+        else if (rep == 2) TA_LAUNCH(N, 2, 1, P);                             \
+        else if (nv == 4) TA_LAUNCH(N, 1, 4, P);                              \
+        else if (nv == 2) TA_LAUNCH(N, 1, 2, P);                              \
+        else TA_LAUNCH(N, 1, 1, P);                                           \
+        launched = true;                                                      \
+    }
+
+template <typename TT>
+static int talk_attn_dispatch(const void* q, long q_tok, const void* k_cache,
+                              const void* v_cache, const int* block_table,
+                              int bt_stride, const int* positions,
+                              const int* seq_idx, float* part_acc,
+                              float* part_ml, int splits, int Tn, int H,
+                              int G, int D, int Dv, int bs, int window,
+                              hipStream_t s) {
+    const bool pair = Dv % 2 == 0;
+    int dpl = pair ? 2 * ((Dv + 2 * WAVE - 1) / (2 * WAVE))
+                   : (Dv + WAVE - 1) / WAVE;
+    if (dpl == 3) dpl = 4;
+    const int group = H / G;
+    const int rep = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
+    // value heads per wave: scores are recomputed per block of value heads
+    const int nv = G >= 4 ? 4 : G >= 2 ? 2 : 1;
+    const int units = H / rep;
+    const int vblocks = (G + nv - 1) / nv;
+    const size_t smem = (size_t)SA_WAVES * rep * D * sizeof(float);
+    const dim3 grid(Tn, (units * vblocks + SA_WAVES - 1) / SA_WAVES, splits);
+    bool launched = false;
+    TA_CASE(2, true) TA_CASE(4, true)
+    TA_CASE(1, false) TA_CASE(2, false) TA_CASE(4, false)
+    return launched ? 0 : 1;
+}
+
+// Scores and per-value-head sums into the partial buffers; nonzero when a
+// head size exceeds 256.
+extern "C" int launch_talk_attn(const void* q, long q_tok,
+                                const void* k_cache, const void* v_cache,
+                                const int* block_table, int bt_stride,
+                                const int* positions, const int* seq_idx,
+                                float* part_acc, float* part_ml, int splits,
+                                int Tn, int H, int G, int D, int Dv, int bs,
+                                int window, int f32, hipStream_t s) {
+    if (D > SA_MAXD || Dv > SA_MAXD) return 1;
+    if (Tn == 0) return 0;
+    if (f32)
+        return talk_attn_dispatch<float>(
+            q, q_tok, k_cache, v_cache, block_table, bt_stride, positions,
+            seq_idx, part_acc, part_ml, splits, Tn, H, G, D, Dv, bs, window,
+            s);
+    return talk_attn_dispatch<unsigned short>(
+        q, q_tok, k_cache, v_cache, block_table, bt_stride, positions,
+        seq_idx, part_acc, part_ml, splits, Tn, H, G, D, Dv, bs, window, s);
+}
+
+// Split merge + head mix + sigmoid gate -> out; nonzero when the LDS need
+// exceeds 64 KB.
+extern "C" int launch_talk_mix(const float* part_acc, const float* part_ml,
+                               const float* talk, const void* gate,
+                               long gate_tok, void* out, long out_tok,
+                               int splits, int Tn, int H, int G, int Dv,
+                               int f32, hipStream_t s) {
+    if (Tn == 0) return 0;
+    const size_t smem =
+        ((size_t)splits * H + (size_t)H * H + (size_t)H * Dv) * sizeof(float);
+    if (smem > 64 * 1024) return 1;
+    if (f32)
+        talk_mix_kernel<float><<<Tn, 256, smem, s>>>(
+            part_acc, part_ml, talk, (const float*)gate, gate_tok,
+            (float*)out, out_tok, splits, Tn, H, G, Dv);
+    else
+        talk_mix_kernel<unsigned short><<<Tn, 256, smem, s>>>(
+            part_acc, part_ml, talk, (const unsigned short*)gate, gate_tok,
+            (unsigned short*)out, out_tok, splits, Tn, H, G, Dv);
+    return 0;
+}

@@ -27,6 +27,8 @@ ext = CUDAExtension(
         os.path.join(CSRC, "hybrid_ext.cpp"),
         os.path.join(CSRC, "hybrid.hip"),
         os.path.join(CSRC, "mixers.hip"),
+        os.path.join(CSRC, "sandwich_ext.cpp"),
+        os.path.join(CSRC, "sandwich.hip"),
     ],
     extra_compile_args={
         "cxx": ["-O3", "-std=c++17"]
