@@ -495,7 +495,9 @@ extern "C" int launch_attn_prefill_paged_sink(
 // Scores use head h's own key head. window > 0: row at absolute position p
 // sees keys p - window < j <= p; key tiles wholly before the tile's first
 // window are skipped. Same tiling and fragment maps as attn_prefill_mfma;
-// the V^T tile is staged once per value head against the same P tile.
+// the V^T tile is staged once per value head against the same P tile. A
+// launch covers the NV value heads from vh0 on (registers hold NV output
+// accumulators); more value heads take further launches.
 template <int HD, int NV>
 __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
     const unsigned short* __restrict__ q,
@@ -503,7 +505,7 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
     const unsigned short* __restrict__ v,  // v_cache [nb,nkv,bs,HD]
     const int* __restrict__ cu, const int* __restrict__ block_table,
     const int* __restrict__ seq_lens, float* __restrict__ part, int nq,
-    int nkv, long s_q, int W, int bs, int window) {
+    int nkv, int vh0, long s_q, int W, int bs, int window) {
     constexpr int KSTEPS = HD / 32;
     const int seq = blockIdx.z;
     const int h = blockIdx.y;
@@ -564,7 +566,7 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
     constexpr int THREADS_PER_ROW = HD / 8;
 
     for (int kb = kb0; kb < kv_end; kb += PF_TN) {
-        // ---- stage K tile [64][HD] (own key head) and V^T of value head 0
+        // ---- stage K tile [64][HD] (own key head) and V^T of value head vh0
         __syncthreads();
         for (int i = tid; i < PF_TN * THREADS_PER_ROW; i += 256) {
             const int key = i / THREADS_PER_ROW;
@@ -574,7 +576,7 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
             if (gk < kv_end) {
                 const long base = (long)bt[gk / bs] * nkv * bs + gk % bs;
                 kraw = load_kv8_bf16(k + (base + (long)kvh * bs) * HD + d);
-                vraw = load_kv8_bf16(v + base * HD + d);
+                vraw = load_kv8_bf16(v + (base + (long)vh0 * bs) * HD + d);
             }
             *reinterpret_cast<bf16x8*>(k_s + key * (HD + PF_PAD) + d) = kraw;
 #pragma unroll
@@ -668,7 +670,7 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
         }
 #pragma unroll
         for (int n = 0; n < NV; ++n) {
-            if (n >= nkv) break;            // uniform over the workgroup
+            if (vh0 + n >= nkv) break;      // uniform over the workgroup
             if (n > 0) {
                 // every wave is done with the previous value head's tile
                 __syncthreads();
@@ -680,7 +682,8 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
                     if (gk < kv_end) {
                         const long base =
                             (long)bt[gk / bs] * nkv * bs + gk % bs;
-                        vraw = load_kv8_bf16(v + (base + (long)n * bs) * HD + d);
+                        vraw = load_kv8_bf16(
+                            v + (base + (long)(vh0 + n) * bs) * HD + d);
                     }
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
@@ -712,8 +715,9 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
         const float inv = (l_run[r] > 0.f) ? 1.f / l_run[r] : 0.f;
 #pragma unroll
         for (int n = 0; n < NV; ++n) {
-            if (n >= nkv) break;
-            float* orow = part + (((long)(s0 + qrow) * nq + h) * nkv + n) * HD;
+            if (vh0 + n >= nkv) break;
+            float* orow =
+                part + (((long)(s0 + qrow) * nq + h) * nkv + vh0 + n) * HD;
 #pragma unroll
             for (int nb = 0; nb < HD / 16; ++nb)
                 orow[nb * 16 + li] = o_acc[n][nb][r] * inv;
@@ -723,14 +727,14 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
 
 // Packed bf16 query chunks against the paged history, each query head's
 // softmax weights applied to every value head: part [T, nq, nkv, hd] fp32.
-// Head size 64 or 128 and nkv <= 4 (returns nonzero otherwise); every score
-// multiplier is already in q.
+// Head size 64 or 128 (returns nonzero otherwise); every score multiplier
+// is already in q.
 extern "C" int launch_attn_prefill_paged_cross(
     const unsigned short* q, long s_q, const unsigned short* k_cache,
     const unsigned short* v_cache, const int* cu, const int* block_table,
     const int* seq_lens, float* part, int nseq, int nq, int nkv, int hd,
     int W, int bs, int max_qlen, int window, hipStream_t stream) {
-    if ((hd != 64 && hd != 128) || nkv > 4 || nkv < 1) return 1;
+    if ((hd != 64 && hd != 128) || nkv < 1) return 1;
     if (nseq == 0 || max_qlen == 0) return 0;
     const int tiles = (max_qlen + PF_TM - 1) / PF_TM;
     dim3 grid(tiles, nq, nseq);
@@ -738,12 +742,18 @@ extern "C" int launch_attn_prefill_paged_cross(
 #define PFC(HDV, NVV)                                                          \
     hipLaunchKernelGGL((attn_prefill_cross_mfma<HDV, NVV>), grid, dim3(256),   \
                        smem, stream, q, k_cache, v_cache, cu, block_table,     \
-                       seq_lens, part, nq, nkv, s_q, W, bs, window)
+                       seq_lens, part, nq, nkv, vh0, s_q, W, bs, window)
     const int nv = nkv > 2 ? 4 : nkv;
-    if (hd == 128) {
-        if (nv == 4) PFC(128, 4); else if (nv == 2) PFC(128, 2); else PFC(128, 1);
-    } else {
-        if (nv == 4) PFC(64, 4); else if (nv == 2) PFC(64, 2); else PFC(64, 1);
+    for (int vh0 = 0; vh0 < nkv; vh0 += nv) {
+        if (hd == 128) {
+            if (nv == 4) PFC(128, 4);
+            else if (nv == 2) PFC(128, 2);
+            else PFC(128, 1);
+        } else {
+            if (nv == 4) PFC(64, 4);
+            else if (nv == 2) PFC(64, 2);
+            else PFC(64, 1);
+        }
     }
 #undef PFC
     return 0;

@@ -233,8 +233,7 @@ void talk_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
     // hi+lo pair) to the values of all key/value heads; single rows of the
     // same step ride along. fp32, other head sizes and pure decode steps
     // take the generic kernel below.
-    if (c == 0 && max_qlen >= 16 && D == Dv && (D == 64 || D == 128) &&
-        G <= 4) {
+    if (c == 0 && max_qlen >= 16 && D == Dv && (D == 64 || D == 128)) {
         const long B = cu.numel() - 1;
         TORCH_CHECK(block_table.size(0) == B);
         Tensor last = cu.slice(0, 1, B + 1).to(torch::kLong) - 1;

@@ -173,6 +173,50 @@ def compare_pugozen(args) -> None:
                                     device, p_batch, p_len, d_batch, d_len)
 
 
+def compare_pimodra(args) -> None:
+    """Prefill and decode throughput of a Pimodra stack (head-mixing
+    windowed GQA attention with rotate-then-unit-norm q/k and an output
+    gate; a dense PolyNorm feed-forward layer followed by a block of
+    group-routed expert layers that runs twice with shared tensors; grouped
+    weighted norms around every sublayer, fp32 residual) beside the closest
+    stack the framework already served: GQA attention + routed experts at
+    equal width, layer runs, head count/size, key/value heads and expert
+    sizes. The window (4096) covers every context here, so both models
+    attend the same keys. Random weights, synthetic prompts, one GPU."""
+    from bee2bee_amd.models.hybrid import pimodra_layers
+    from bee2bee_amd.models.spec import ModelSpec, hybrid_spec
+
+    on_gpu = torch.cuda.is_available()
+    device = "cuda:0" if on_gpu else "cpu"
+    vocab, head_dim = 32000, 128
+    p_batch, p_len = 8, (2048 if on_gpu else 48)
+    d_batch, d_len = (64 if on_gpu else 4), (1024 if on_gpu else 32)
+    for size in args.compare_pimodra.split(","):
+        z = HYBRID_SIZES[size.strip()]
+        W, H, ff, E = z["width"], z["heads"], z["ff"], z["experts"]
+        if not on_gpu:
+            W, H, head_dim, vocab, ff, E = 64, 4, 16, 256, 32, 4
+        # 4 checkpoint layers, layers 1..2 run twice: 6 layer runs
+        layers = pimodra_layers(
+            4, W, heads=H, kv_heads=max(1, H // 4), dim=head_dim,
+            window=4096, ff=2 * ff, experts=E, top_k=2, expert_ff=ff,
+            groups=4, keep=2, moe_from=1, loop=(1, 3, 2))
+        pm = hybrid_spec(
+            f"pimodra-{size}", vocab, W, layers, eps=1e-6, embed_scale=1.0,
+            canon_taps=0, max_seq_len=8192, arch="pimodra",
+            norm_type="group_rmsnorm", act_type="polynorm")
+        pm.tie_embeddings, pm.norm_groups, pm.step_rows = True, 2, 2
+        pm.n_kv_heads = max(1, H // 4)
+        dense = ModelSpec(
+            name=f"gqa-moe-{size}", vocab_size=vocab, hidden_size=W,
+            intermediate_size=ff, n_layers=len(layers), n_heads=H,
+            n_kv_heads=max(1, H // 4), head_dim=head_dim, rope_theta=1e6,
+            max_seq_len=8192, n_experts=E, top_k_experts=2)
+        for spec in (pm, dense):
+            _measure_prefill_decode(spec, "pimodra-vs-dense", size, args,
+                                    device, p_batch, p_len, d_batch, d_len)
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -200,6 +244,15 @@ def main() -> None:
                          "beside a dense GQA transformer of equal width, "
                          "depth and heads, at the comma-separated sizes "
                          "(s, m, l); one JSON line per size and model")
+    ap.add_argument("--compare-pimodra", default=None, metavar="SIZES",
+                    help="instead of the headline run: prefill and decode "
+                         "throughput of the Pimodra stack (head-mixing "
+                         "windowed attention, PolyNorm and group-routed "
+                         "expert feed-forwards, a repeated block) beside a "
+                         "GQA-attention MoE stack of equal width, layer "
+                         "runs, heads and expert sizes, at the "
+                         "comma-separated sizes (s, m, l); one JSON line "
+                         "per size and model")
     ap.add_argument("--preflight", action="store_true",
                     help="run the scale-run preflight checks (RCCL self-"
                          "test, master endpoint, env, rank wiring) and exit")
@@ -219,6 +272,9 @@ def main() -> None:
         return
     if args.compare_pugozen:
         compare_pugozen(args)
+        return
+    if args.compare_pimodra:
+        compare_pimodra(args)
         return
 
     from bee2bee_amd.models.spec import resolve_spec

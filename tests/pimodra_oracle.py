@@ -206,3 +206,95 @@ def forward(cfg: dict, tensors: Dict[str, torch.Tensor], tokens: List[int],
             taps.append(x.clone())
     x = group_norm(x, tensors["final.norm"].to(F64), groups, eps)
     return x @ embed.T
+
+
+# ------------------------------------------------ small random checkpoints
+
+def make_config(vocab=97, width=24, groups=2, eps=1e-6, heads=4, kv_heads=2,
+                dim=6, vdim=10, window=9, rot_dims=4, scaling=True,
+                kinds=("dense", "moe", "moe"), ff=20, experts=6, top=2,
+                n_groups=3, keep=2, expert_ff=8, loop=(1, 3, 2)) -> dict:
+    rot = None
+    if rot_dims:
+        rot = {"base": 500.0, "dims": rot_dims}
+        if scaling:
+            rot["scaling"] = {"factor": 3.0, "original": 16, "fast": 4.0,
+                              "slow": 0.5}
+    layers = []
+    for kind in kinds:
+        mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim,
+                 "vdim": vdim, "scale": 1.7 / math.sqrt(dim)}
+        if window:
+            mixer["mask"] = {"size": window}
+        if rot:
+            mixer["rot"] = rot
+        if kind == "dense":
+            mlp = {"kind": "dense", "ff": ff}
+        elif kind == "moe":
+            mlp = {"kind": "moe", "expert": {"ff": expert_ff},
+                   "router": {"experts": experts, "top": top,
+                              "groups": {"count": n_groups, "keep": keep}}}
+        else:
+            mlp = None
+        layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+    cfg = {"architecture": "Pimodra", "vocab": vocab, "width": width,
+           "norm": {"eps": eps, "groups": groups}, "layers": layers}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
+def random_weights(cfg: dict, seed: int = 0) -> Dict[str, torch.Tensor]:
+    """bf16 tensors under the checkpoint's names."""
+    g = torch.Generator().manual_seed(seed)
+    W = int(cfg["width"])
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return (mean + std * torch.randn(*shape, generator=g)).bfloat16()
+
+    T = {"embed": rnd(cfg["vocab"], W), "final.norm": rnd(W, std=0.1, mean=1.0)}
+    if cfg.get("loop"):
+        T["loop.step"] = rnd(int(cfg["loop"]["times"]), W, std=0.5)
+    for i, l in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", l["mixer"]
+        H, G = m["heads"], m.get("kv_heads", m["heads"])
+        D, Dv = m["dim"], m["vdim"]
+        for n in ("norm1", "norm1b"):
+            T[p + n] = rnd(W, std=0.1, mean=1.0)
+        T[p + "mix.q"] = rnd(H * D, W, std=W ** -0.5)
+        T[p + "mix.k"] = rnd(G * D, W, std=W ** -0.5)
+        T[p + "mix.v"] = rnd(G * Dv, W, std=W ** -0.5)
+        T[p + "mix.g"] = rnd(H * Dv, W, std=W ** -0.5)
+        T[p + "mix.o"] = rnd(W, H * Dv, std=(H * Dv) ** -0.5)
+        T[p + "mix.talk"] = (torch.eye(H) + 0.3 * torch.randn(
+            H, H, generator=g)).bfloat16()
+        f = l.get("mlp")
+        if not f:
+            continue
+        for n in ("norm2", "norm2b"):
+            T[p + n] = rnd(W, std=0.1, mean=1.0)
+        if f["kind"] == "dense":
+            T[p + "mlp.up"] = rnd(f["ff"], W, std=W ** -0.5)
+            T[p + "mlp.down"] = rnd(W, f["ff"], std=f["ff"] ** -0.5)
+            T[p + "mlp.act"] = rnd(4, std=0.3, mean=0.3)
+        else:
+            ff = f["expert"]["ff"]
+            T[p + "mlp.router"] = rnd(f["router"]["experts"], W, std=1.5 * W ** -0.5)
+            for e in range(f["router"]["experts"]):
+                T[f"{p}mlp.e{e}.gate"] = rnd(ff, W, std=W ** -0.5)
+                T[f"{p}mlp.e{e}.up"] = rnd(ff, W, std=W ** -0.5)
+                T[f"{p}mlp.e{e}.down"] = rnd(W, ff, std=ff ** -0.5)
+    return T
+
+
+def save_checkpoint(path: str, cfg: dict, tensors: Dict[str, torch.Tensor]):
+    import json
+    import os
+
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    save_file({k: v.contiguous() for k, v in tensors.items()},
+              os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)

@@ -117,12 +117,12 @@ def test_talk_attn_decode_splits(dtype):
 
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("G,window", [(1, 0), (2, 100), (4, 64), (2, 1),
-                                      (3, 300)])
+                                      (3, 300), (8, 40), (6, 0)])
 def test_talk_attn_matrix_core(D, G, window):
     """bf16 prompt portions of head size 64/128: the query-tiled kernel;
     chunks with history, a chunk shorter than a tile, single rows riding
     along, windows that end inside, at and before a key tile"""
-    H = G * 2 if G != 3 else 6
+    H = G * 2
     a, b = _attn_case(torch.bfloat16, [70, 1, 130, 16, 1],
                       [0, 200, 57, 500, 0], H, G, D, D, window, 32, seed=3)
     torch.testing.assert_close(a, b, rtol=2e-2, atol=4e-2)
