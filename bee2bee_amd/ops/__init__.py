@@ -449,14 +449,17 @@ def rope_unit_store(q, k, v, eps: float, rope_dims: int, positions, cos, sin,
 
 def talk_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
               cu_seqlens, talk, gate, window: int, out,
-              max_qlen: int = 0) -> None:
+              max_qlen: int = 0, path: str = "auto") -> None:
     """max_qlen: longest chunk of the step (host int); with bf16 pages, a
     matrix-core head size and a chunk of at least 16 rows the step takes
-    the query-tiled kernel."""
+    the query-tiled kernel. path (GPU only): "auto", or force "scored"
+    (scores written once, heads mixed before the values are read) or
+    "cross" (every head's weights against every value head, mixed after)."""
     if _use_hip(q):
         require_hip().talk_attn(q, k_cache, v_cache, block_table, positions,
                                 seq_idx, cu_seqlens, talk, gate, window, out,
-                                max_qlen)
+                                max_qlen,
+                                {"auto": 0, "scored": 1, "cross": 2}[path])
         return
     reference.talk_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
                         cu_seqlens, talk, gate, window, out)

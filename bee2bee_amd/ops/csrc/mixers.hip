@@ -1583,9 +1583,11 @@ talk_attn_kernel(const T* __restrict__ q, long q_tok,
     }
 }
 
-// Merge of the key splits + head mix + output gate. Workgroup per token.
+// Merge of the key splits + head mix + output gate. Workgroup per (token,
+// key/value head c): the merged, normalized sums A[g, c] of all query heads
+// g are staged in LDS, then every query head of group c takes its mixture.
 // part_ml == nullptr: the partials are already normalized (one split).
-// LDS: wts [S*H] | talk [H*H] | A_c [H*Dv].
+// LDS: wts [S*H] | talk rows of the group [rep*H] | A_c [H*Dv].
 template <typename T>
 __global__ void __launch_bounds__(256)
 talk_mix_kernel(const float* __restrict__ part_acc,
@@ -1594,11 +1596,11 @@ talk_mix_kernel(const float* __restrict__ part_acc,
                 long gate_tok, T* __restrict__ out, long out_tok, int splits,
                 int Tn, int H, int G, int Dv) {
     extern __shared__ __attribute__((aligned(16))) float tm_s[];
+    const int rep = H / G;
     float* wts = tm_s;
     float* tk = wts + splits * H;
-    float* A = tk + H * H;
-    const int t = blockIdx.x;
-    const int rep = H / G;
+    float* A = tk + rep * H;
+    const int t = blockIdx.x, c = blockIdx.y;
     for (int h = threadIdx.x; h < H; h += blockDim.x) {
         if (!part_ml) {
             wts[h] = 1.f;
@@ -1620,33 +1622,331 @@ talk_mix_kernel(const float* __restrict__ part_acc,
         const float rcp = L > 0.f ? 1.f / L : 0.f;
         for (int s = 0; s < splits; ++s) wts[s * H + h] *= rcp;
     }
-    for (int i = threadIdx.x; i < H * H; i += blockDim.x) tk[i] = talk[i];
+    for (int i = threadIdx.x; i < rep * H; i += blockDim.x)
+        tk[i] = talk[(long)c * rep * H + i];
     __syncthreads();
-    for (int c = 0; c < G; ++c) {
-        for (int idx = threadIdx.x; idx < H * Dv; idx += blockDim.x) {
-            const int gq = idx / Dv, d = idx - gq * Dv;
-            float a = 0.f;
-            for (int s = 0; s < splits; ++s)
-                a += wts[s * H + gq] *
-                     part_acc[((((long)s * Tn + t) * H + gq) * G + c) * Dv + d];
-            A[idx] = a;
-        }
-        __syncthreads();
-        for (int idx = threadIdx.x; idx < rep * Dv; idx += blockDim.x) {
-            const int hl = idx / Dv, d = idx - hl * Dv;
-            const int h = c * rep + hl;
-            float o = 0.f;
-            for (int gq = 0; gq < H; ++gq) o += tk[h * H + gq] * A[gq * Dv + d];
-            const float gt =
-                ldf(gate + (long)t * gate_tok + (long)h * Dv + d);
-            stf(out + (long)t * out_tok + (long)h * Dv + d,
-                o / (1.f + expf(-gt)));
-        }
-        __syncthreads();
+    for (int idx = threadIdx.x; idx < H * Dv; idx += blockDim.x) {
+        const int gq = idx / Dv, d = idx - gq * Dv;
+        float a = 0.f;
+        for (int s = 0; s < splits; ++s)
+            a += wts[s * H + gq] *
+                 part_acc[((((long)s * Tn + t) * H + gq) * G + c) * Dv + d];
+        A[idx] = a;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < rep * Dv; idx += blockDim.x) {
+        const int hl = idx / Dv, d = idx - hl * Dv;
+        const int h = c * rep + hl;
+        float o = 0.f;
+        for (int gq = 0; gq < H; ++gq) o += tk[hl * H + gq] * A[gq * Dv + d];
+        const float gt = ldf(gate + (long)t * gate_tok + (long)h * Dv + d);
+        stf(out + (long)t * out_tok + (long)h * Dv + d, o / (1.f + expf(-gt)));
     }
 }
 
 }  // namespace
+
+// ---------------------------------------------------------------------------
+// The same attention for steps whose score matrix is small (decode rows,
+// short portions, windows): the raw scores of every (token, head, visible
+// key) are written once (kernel 1, with the per-split max/sum), and kernel
+// 2 turns them into normalized weights of ALL heads, mixes them with the
+// wave's rows of `talk` — w'_h(j) = sum_g talk[h, g] w_g(j) — and applies
+// the mixed weights to the values of the wave's own key/value head only:
+// each cached value row is read once per key group, as in plain attention.
+// scores [Tn, H, ctx] fp32, entry (j - lo) of a row whose first visible
+// key is lo. Wave layout as above: (token, REP query heads of one key
+// group, key split); lane = key for scores and weights, lane = coordinate
+// pair for the value sum.
+namespace {
+
+template <typename T, int REP>
+__global__ void __launch_bounds__(SA_WAVES * WAVE)
+talk_scores_kernel(const T* __restrict__ q, long q_tok,
+                   const T* __restrict__ k_cache,
+                   const int* __restrict__ block_table, int bt_stride,
+                   const int* __restrict__ positions,
+                   const int* __restrict__ seq_idx,
+                   float* __restrict__ scores, long ctx,
+                   float* __restrict__ part_ml, int Tn, int H, int G, int D,
+                   int bs, int window) {
+    extern __shared__ __attribute__((aligned(16))) float sa_q[];
+    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int t = blockIdx.x;
+    const int unit = blockIdx.y * SA_WAVES + wid;
+    if (unit * REP >= H) return;      // no workgroup barrier below
+    const int h0 = unit * REP;
+    const int split = blockIdx.z, nsplit = gridDim.z;
+    const int p = positions[t];
+    const int g = h0 / (H / G);
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int per =
+        ((p + 1 - lo + nsplit - 1) / nsplit + WAVE - 1) / WAVE * WAVE;
+    const int klo = lo + split * per, khi = min(p + 1, klo + per);
+    float* qv = sa_q + (long)wid * REP * D;
+    for (int i = lane; i < REP * D; i += WAVE)
+        qv[i] = ldf(q + (long)t * q_tok + (long)h0 * D + i);
+    WAVE_LDS_SYNC();
+    const int* bt = block_table + (long)seq_idx[t] * bt_stride;
+    float m[REP], l[REP];
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+        m[r] = -INFINITY;
+        l[r] = 0.f;
+    }
+    for (int j0 = klo; j0 < khi; j0 += WAVE) {
+        const int j = j0 + lane;
+        const bool valid = j < khi;
+        float sc[REP];
+#pragma unroll
+        for (int r = 0; r < REP; ++r) sc[r] = 0.f;
+        if (valid) {
+            const int row = (bt[j / bs] * G + g) * bs + j % bs;
+            SaDots<T, REP>::run(k_cache + (long)row * D, qv, D, sc);
+        }
+#pragma unroll
+        for (int r = 0; r < REP; ++r) {
+            const float sv = valid ? sc[r] : -INFINITY;
+            if (valid)
+                scores[((long)t * H + h0 + r) * ctx + (j - lo)] = sv;
+            const float m_new = fmaxf(m[r], wave_max(sv));
+            const float e = valid ? expf(sv - m_new) : 0.f;
+            l[r] = l[r] * expf(m[r] - m_new) + wave_sum(e);
+            m[r] = m_new;
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < REP; ++r) {
+            const long prow = ((long)split * Tn + t) * H + h0 + r;
+            part_ml[prow * 2] = m[r];
+            part_ml[prow * 2 + 1] = l[r];
+        }
+    }
+}
+
+// ml_splits: the number of key splits kernel 1 ran with (rows of part_ml).
+// Per-wave LDS: max [H] | 1/sum [H] | talk rows [REP*H].
+template <typename T, int DPL, int REP, bool PAIR>
+__global__ void __launch_bounds__(SA_WAVES * WAVE)
+talk_pv_kernel(const float* __restrict__ scores, long ctx,
+               const float* __restrict__ part_ml, int ml_splits,
+               const float* __restrict__ talk,
+               const T* __restrict__ v_cache,
+               const int* __restrict__ block_table, int bt_stride,
+               const int* __restrict__ positions,
+               const int* __restrict__ seq_idx, const T* __restrict__ gate,
+               long gate_tok, T* __restrict__ out, long out_tok,
+               float* __restrict__ part_o, int Tn, int H, int G, int Dv,
+               int bs, int window) {
+    extern __shared__ __attribute__((aligned(16))) float tp_s[];
+    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int t = blockIdx.x;
+    const int unit = blockIdx.y * SA_WAVES + wid;
+    if (unit * REP >= H) return;      // no workgroup barrier below
+    const int h0 = unit * REP;
+    const int split = blockIdx.z, nsplit = gridDim.z;
+    const int p = positions[t];
+    const int g = h0 / (H / G);
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int per =
+        ((p + 1 - lo + nsplit - 1) / nsplit + WAVE - 1) / WAVE * WAVE;
+    const int klo = lo + split * per, khi = min(p + 1, klo + per);
+    float* Mh = tp_s + (long)wid * (2 + REP) * H;
+    float* iL = Mh + H;
+    float* tkw = iL + H;
+    for (int h = lane; h < H; h += WAVE) {
+        float M = -INFINITY;
+        for (int s = 0; s < ml_splits; ++s) {
+            const long row = ((long)s * Tn + t) * H + h;
+            if (part_ml[row * 2 + 1] > 0.f) M = fmaxf(M, part_ml[row * 2]);
+        }
+        float L = 0.f;
+        for (int s = 0; s < ml_splits; ++s) {
+            const long row = ((long)s * Tn + t) * H + h;
+            const float l = part_ml[row * 2 + 1];
+            if (l > 0.f) L += l * expf(part_ml[row * 2] - M);
+        }
+        Mh[h] = M;
+        iL[h] = L > 0.f ? 1.f / L : 0.f;
+    }
+    for (int i = lane; i < REP * H; i += WAVE)
+        tkw[i] = talk[(long)h0 * H + i];
+    WAVE_LDS_SYNC();
+    const int* bt = block_table + (long)seq_idx[t] * bt_stride;
+    float acc[REP][DPL];
+#pragma unroll
+    for (int r = 0; r < REP; ++r)
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) acc[r][i] = 0.f;
+    const float* srow = scores + (long)t * H * ctx;
+    for (int j0 = klo; j0 < khi; j0 += WAVE) {
+        const int j = j0 + lane;
+        const bool valid = j < khi;
+        const int nk = min(WAVE, khi - j0);
+        int row = 0;            // lanes past the end point at a real row
+        float pj[REP];
+#pragma unroll
+        for (int r = 0; r < REP; ++r) pj[r] = 0.f;
+        if (valid) {
+            row = (bt[j / bs] * G + g) * bs + j % bs;
+            for (int gq = 0; gq < H; ++gq) {
+                const float e =
+                    expf(srow[(long)gq * ctx + (j - lo)] - Mh[gq]) * iL[gq];
+#pragma unroll
+                for (int r = 0; r < REP; ++r) pj[r] += tkw[r * H + gq] * e;
+            }
+        }
+#pragma unroll 2
+        for (int jj = 0; jj < nk; jj += SA_PV) {
+            float vv[SA_PV][DPL];
+#pragma unroll
+            for (int x = 0; x < SA_PV; ++x) {
+                const T* vr =
+                    v_cache + (long)__builtin_amdgcn_readlane(row, jj + x) * Dv;
+                if constexpr (PAIR) {
+#pragma unroll
+                    for (int i = 0; i < DPL; i += 2) {
+                        const int d = sa_coord<true>(lane, i);
+                        vv[x][i] = vv[x][i + 1] = 0.f;
+                        if (d < Dv) sa_ld2(vr + d, vv[x][i], vv[x][i + 1]);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < DPL; ++i) {
+                        const int d = sa_coord<false>(lane, i);
+                        vv[x][i] = d < Dv ? ldf(vr + d) : 0.f;
+                    }
+                }
+            }
+#pragma unroll
+            for (int x = 0; x < SA_PV; ++x)
+#pragma unroll
+                for (int r = 0; r < REP; ++r) {
+                    const float pb = __builtin_bit_cast(
+                        float, __builtin_amdgcn_readlane(
+                                   __builtin_bit_cast(int, pj[r]), jj + x));
+#pragma unroll
+                    for (int i = 0; i < DPL; ++i) acc[r][i] += pb * vv[x][i];
+                }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+        const int h = h0 + r;
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) {
+            const int d = sa_coord<PAIR>(lane, i);
+            if (d >= Dv) continue;
+            if (nsplit == 1) {
+                const float gt =
+                    ldf(gate + (long)t * gate_tok + (long)h * Dv + d);
+                stf(out + (long)t * out_tok + (long)h * Dv + d,
+                    acc[r][i] / (1.f + expf(-gt)));
+            } else {
+                part_o[(((long)split * Tn + t) * H + h) * Dv + d] = acc[r][i];
+            }
+        }
+    }
+}
+
+// out = sigmoid(gate) * sum over splits of part_o [S, Tn, H*Dv]
+template <typename T>
+__global__ void talk_sum_gate_kernel(const float* __restrict__ part_o,
+                                     const T* __restrict__ gate, long gate_tok,
+                                     T* __restrict__ out, long out_tok,
+                                     int splits, int Tn, int N) {
+    const int t = blockIdx.x;
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < N;
+         i += gridDim.y * blockDim.x) {
+        float a = 0.f;
+        for (int s = 0; s < splits; ++s)
+            a += part_o[((long)s * Tn + t) * N + i];
+        const float gt = ldf(gate + (long)t * gate_tok + i);
+        stf(out + (long)t * out_tok + i, a / (1.f + expf(-gt)));
+    }
+}
+
+}  // namespace
+
+#define TP_LAUNCH(N, R, P)                                                    \
+    talk_pv_kernel<TT, N, R, P><<<grid, SA_WAVES * WAVE, smem2, s>>>(         \
+        scores, ctx, part_ml, splits, talk, (const TT*)v_cache, block_table,  \
+        bt_stride, positions, seq_idx, (const TT*)gate, gate_tok, (TT*)out,   \
+        out_tok, part_o, Tn, H, G, Dv, bs, window)
+
+#define TP_CASE(N, P)                                                         \
+    if (dpl == N && pair == P) {                                              \
+        if (rep == 4) TP_LAUNCH(N, 4, P);                                     \
+        else if (rep == 2) TP_LAUNCH(N, 2, P);                                \
+        else TP_LAUNCH(N, 1, P);                                              \
+        launched = true;                                                      \
+    }
+
+template <typename TT>
+static int talk_scored_dispatch(const void* q, long q_tok, const void* k_cache,
+                                const void* v_cache, const int* block_table,
+                                int bt_stride, const int* positions,
+                                const int* seq_idx, const float* talk,
+                                const void* gate, long gate_tok, void* out,
+                                long out_tok, float* scores, long ctx,
+                                float* part_ml, float* part_o, int splits,
+                                int Tn, int H, int G, int D, int Dv, int bs,
+                                int window, hipStream_t s) {
+    const bool pair = Dv % 2 == 0;
+    int dpl = pair ? 2 * ((Dv + 2 * WAVE - 1) / (2 * WAVE))
+                   : (Dv + WAVE - 1) / WAVE;
+    if (dpl == 3) dpl = 4;
+    const int group = H / G;
+    const int rep = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
+    const int units = H / rep;
+    const dim3 grid(Tn, (units + SA_WAVES - 1) / SA_WAVES, splits);
+    const size_t smem1 = (size_t)SA_WAVES * rep * D * sizeof(float);
+    const size_t smem2 = (size_t)SA_WAVES * (2 + rep) * H * sizeof(float);
+#define TS_LAUNCH(R)                                                          \
+    talk_scores_kernel<TT, R><<<grid, SA_WAVES * WAVE, smem1, s>>>(           \
+        (const TT*)q, q_tok, (const TT*)k_cache, block_table, bt_stride,      \
+        positions, seq_idx, scores, ctx, part_ml, Tn, H, G, D, bs, window)
+    if (rep == 4) TS_LAUNCH(4);
+    else if (rep == 2) TS_LAUNCH(2);
+    else TS_LAUNCH(1);
+#undef TS_LAUNCH
+    bool launched = false;
+    TP_CASE(2, true) TP_CASE(4, true)
+    TP_CASE(1, false) TP_CASE(2, false) TP_CASE(4, false)
+    if (!launched) return 1;
+    if (splits > 1) {
+        const int N = H * Dv;
+        const dim3 g2(Tn, (N + 255) / 256);
+        talk_sum_gate_kernel<TT><<<g2, 256, 0, s>>>(
+            part_o, (const TT*)gate, gate_tok, (TT*)out, out_tok, splits, Tn,
+            N);
+    }
+    return 0;
+}
+
+// Scores written once, then mixed weights against each head's own values.
+// scores [Tn, H, ctx], part_ml [splits, Tn, H, 2], part_o [splits, Tn, H,
+// Dv] (unused when splits == 1); nonzero when a head size exceeds 256.
+extern "C" int launch_talk_attn_scored(
+    const void* q, long q_tok, const void* k_cache, const void* v_cache,
+    const int* block_table, int bt_stride, const int* positions,
+    const int* seq_idx, const float* talk, const void* gate, long gate_tok,
+    void* out, long out_tok, float* scores, long ctx, float* part_ml,
+    float* part_o, int splits, int Tn, int H, int G, int D, int Dv, int bs,
+    int window, int f32, hipStream_t s) {
+    if (D > SA_MAXD || Dv > SA_MAXD) return 1;
+    if (Tn == 0) return 0;
+    if (f32)
+        return talk_scored_dispatch<float>(
+            q, q_tok, k_cache, v_cache, block_table, bt_stride, positions,
+            seq_idx, talk, gate, gate_tok, out, out_tok, scores, ctx, part_ml,
+            part_o, splits, Tn, H, G, D, Dv, bs, window, s);
+    return talk_scored_dispatch<unsigned short>(
+        q, q_tok, k_cache, v_cache, block_table, bt_stride, positions,
+        seq_idx, talk, gate, gate_tok, out, out_tok, scores, ctx, part_ml,
+        part_o, splits, Tn, H, G, D, Dv, bs, window, s);
+}
 
 #define TA_LAUNCH(N, R, V, P)                                                 \
     talk_attn_kernel<TT, N, R, V, P><<<grid, SA_WAVES * WAVE, smem, s>>>(     \
@@ -1723,15 +2023,16 @@ extern "C" int launch_talk_mix(const float* part_acc, const float* part_ml,
                                int splits, int Tn, int H, int G, int Dv,
                                int f32, hipStream_t s) {
     if (Tn == 0) return 0;
-    const size_t smem =
-        ((size_t)splits * H + (size_t)H * H + (size_t)H * Dv) * sizeof(float);
+    const size_t smem = ((size_t)splits * H + (size_t)(H / G) * H +
+                         (size_t)H * Dv) * sizeof(float);
     if (smem > 64 * 1024) return 1;
+    const dim3 grid(Tn, G);
     if (f32)
-        talk_mix_kernel<float><<<Tn, 256, smem, s>>>(
+        talk_mix_kernel<float><<<grid, 256, smem, s>>>(
             part_acc, part_ml, talk, (const float*)gate, gate_tok,
             (float*)out, out_tok, splits, Tn, H, G, Dv);
     else
-        talk_mix_kernel<unsigned short><<<Tn, 256, smem, s>>>(
+        talk_mix_kernel<unsigned short><<<grid, 256, smem, s>>>(
             part_acc, part_ml, talk, (const unsigned short*)gate, gate_tok,
             (unsigned short*)out, out_tok, splits, Tn, H, G, Dv);
     return 0;

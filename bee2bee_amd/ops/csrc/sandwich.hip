@@ -22,6 +22,39 @@ template <> DEV_INLINE void stf<unsigned short>(unsigned short* p, float v) {
     *p = f2bf(v);
 }
 
+// VEC consecutive elements <-> floats. VEC = 4 moves 16 B (fp32) or 8 B
+// (bf16) per lane and needs rows whose length is a multiple of 4.
+template <typename T, int VEC> DEV_INLINE void ldv(const T* p, float* o);
+template <> DEV_INLINE void ldv<float, 1>(const float* p, float* o) { o[0] = *p; }
+template <> DEV_INLINE void ldv<unsigned short, 1>(const unsigned short* p, float* o) {
+    o[0] = bf2f(*p);
+}
+template <> DEV_INLINE void ldv<float, 4>(const float* p, float* o) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+    o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
+}
+template <> DEV_INLINE void ldv<unsigned short, 4>(const unsigned short* p, float* o) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    o[0] = bf2f((unsigned short)(w.x & 0xffffu));
+    o[1] = bf2f((unsigned short)(w.x >> 16));
+    o[2] = bf2f((unsigned short)(w.y & 0xffffu));
+    o[3] = bf2f((unsigned short)(w.y >> 16));
+}
+template <typename T, int VEC> DEV_INLINE void stv(T* p, const float* o);
+template <> DEV_INLINE void stv<float, 1>(float* p, const float* o) { *p = o[0]; }
+template <> DEV_INLINE void stv<unsigned short, 1>(unsigned short* p, const float* o) {
+    *p = f2bf(o[0]);
+}
+template <> DEV_INLINE void stv<float, 4>(float* p, const float* o) {
+    *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+}
+template <> DEV_INLINE void stv<unsigned short, 4>(unsigned short* p, const float* o) {
+    uint2 w;
+    w.x = (unsigned int)f2bf(o[0]) | ((unsigned int)f2bf(o[1]) << 16);
+    w.y = (unsigned int)f2bf(o[2]) | ((unsigned int)f2bf(o[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = w;
+}
+
 constexpr int GN_MAXG = 64;     // parts of a row
 constexpr int GN_MAXW = 16;     // waves per workgroup
 
@@ -58,7 +91,8 @@ DEV_INLINE void group_sumsq(const float* buf, int W, int groups, float* red,
 // gnorm: each of `groups` equal consecutive parts of the row divided by its
 // own sqrt(mean^2 + eps). One workgroup per row; the row (and y) are held
 // in LDS between the passes, so every operand crosses HBM once.
-template <typename YT, typename OT>
+// VEC = 4 needs the part width (W / groups) to be a multiple of 4.
+template <typename YT, typename OT, int VEC>
 __global__ void add_group_rmsnorm_kernel(float* __restrict__ resid,
                                          const YT* __restrict__ y,
                                          const float* __restrict__ w_post,
@@ -76,27 +110,46 @@ __global__ void add_group_rmsnorm_kernel(float* __restrict__ resid,
     float* rr = resid + t * (long)W;
     if (y) {
         const YT* yr = y + t * (long)W;
-        for (int i = threadIdx.x; i < W; i += blockDim.x) yrow[i] = ldf(yr + i);
+        for (int i = threadIdx.x * VEC; i < W; i += blockDim.x * VEC) {
+            float v[VEC];
+            ldv<YT, VEC>(yr + i, v);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) yrow[i + j] = v[j];
+        }
         __syncthreads();
         group_sumsq(yrow, W, groups, red, sums);
     }
-    for (int i = threadIdx.x; i < W; i += blockDim.x) {
-        float v = rr[i];
+    for (int i = threadIdx.x * VEC; i < W; i += blockDim.x * VEC) {
+        float v[VEC];
+        ldv<float, VEC>(rr + i, v);
         if (y) {
             const float r = 1.f / sqrtf(sums[i / gw] / (float)gw + eps);
-            v += yrow[i] * r * w_post[i];
+            float wv[VEC];
+            ldv<float, VEC>(w_post + i, wv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] += yrow[i + j] * r * wv[j];
         }
-        if (step) v += step[i];
-        if (y || step) rr[i] = v;
-        row[i] = v;
+        if (step) {
+            float sv[VEC];
+            ldv<float, VEC>(step + i, sv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] += sv[j];
+        }
+        if (y || step) stv<float, VEC>(rr + i, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) row[i + j] = v[j];
     }
     if (!out) return;
     __syncthreads();
     group_sumsq(row, W, groups, red, sums);
     OT* orow = out + t * (long)W;
-    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    for (int i = threadIdx.x * VEC; i < W; i += blockDim.x * VEC) {
         const float r = 1.f / sqrtf(sums[i / gw] / (float)gw + eps);
-        stf(orow + i, row[i] * r * w_pre[i]);
+        float v[VEC], wv[VEC];
+        ldv<float, VEC>(w_pre + i, wv);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = row[i + j] * r * wv[j];
+        stv<OT, VEC>(orow + i, v);
     }
 }
 
@@ -257,10 +310,19 @@ extern "C" int launch_add_group_rmsnorm(float* resid, const void* y,
     if (groups < 1 || groups > GN_MAXG || W % groups) return 1;
     if (T == 0) return 0;
     const size_t sh = (size_t)W * sizeof(float) * (y ? 2 : 1);
-    const int th = row_threads(W);
+    const bool vec = (W / groups) % 4 == 0;
+    const int th = row_threads(vec ? W / 4 : W);
 #define AGN(YT, OT)                                                           \
-    add_group_rmsnorm_kernel<YT, OT><<<T, th, sh, s>>>(                       \
-        resid, (const YT*)y, w_post, step, w_pre, (OT*)out, W, groups, eps)
+    do {                                                                      \
+        if (vec)                                                              \
+            add_group_rmsnorm_kernel<YT, OT, 4><<<T, th, sh, s>>>(            \
+                resid, (const YT*)y, w_post, step, w_pre, (OT*)out, W,        \
+                groups, eps);                                                 \
+        else                                                                  \
+            add_group_rmsnorm_kernel<YT, OT, 1><<<T, th, sh, s>>>(            \
+                resid, (const YT*)y, w_post, step, w_pre, (OT*)out, W,        \
+                groups, eps);                                                 \
+    } while (0)
     if (y_f32 && out_f32) AGN(float, float);
     else if (y_f32) AGN(float, unsigned short);
     else if (out_f32) AGN(unsigned short, float);

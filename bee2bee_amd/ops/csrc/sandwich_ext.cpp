@@ -28,6 +28,11 @@ void launch_silu_glu(const void*, void*, long, long, int, hipStream_t);
 int launch_talk_attn(const void*, long, const void*, const void*, const int*,
                      int, const int*, const int*, float*, float*, int, int,
                      int, int, int, int, int, int, int, hipStream_t);
+int launch_talk_attn_scored(const void*, long, const void*, const void*,
+                            const int*, int, const int*, const int*,
+                            const float*, const void*, long, void*, long,
+                            float*, long, float*, float*, int, int, int, int,
+                            int, int, int, int, int, hipStream_t);
 int launch_talk_mix(const float*, const float*, const float*, const void*,
                     long, void*, long, int, int, int, int, int, int,
                     hipStream_t);
@@ -202,7 +207,10 @@ void talk_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
                const Tensor& block_table, const Tensor& positions,
                const Tensor& seq_idx, const Tensor& cu, const Tensor& talk,
                const Tensor& gate, int64_t window, Tensor& out,
-               int64_t max_qlen) {
+               int64_t max_qlen, int64_t path) {
+    // path: 0 = choose by dtype, head size and step shape; 1 = scores
+    // written once, heads mixed before the values; 2 = every head's weights
+    // against every value head, mixed afterwards (generic kernel)
     const int c = act_code(q, "q");
     check_i32(block_table, "block_table");
     check_i32(positions, "positions");
@@ -233,7 +241,8 @@ void talk_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
     // hi+lo pair) to the values of all key/value heads; single rows of the
     // same step ride along. fp32, other head sizes and pure decode steps
     // take the generic kernel below.
-    if (c == 0 && max_qlen >= 16 && D == Dv && (D == 64 || D == 128)) {
+    if (path == 0 && c == 0 && max_qlen >= 16 && D == Dv &&
+        (D == 64 || D == 128)) {
         const long B = cu.numel() - 1;
         TORCH_CHECK(block_table.size(0) == B);
         Tensor last = cu.slice(0, 1, B + 1).to(torch::kLong) - 1;
@@ -261,9 +270,38 @@ void talk_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
     }
     // few rows (decode): split each row's keys over more waves, at least 64
     // keys per share of the longest context the tables can hold
-    const long ctx = window > 0 ? window : block_table.size(1) * (long)bs;
+    const long cap = block_table.size(1) * (long)bs;
+    const long ctx = window > 0 ? std::min<long>(window, cap) : cap;
     const long group = H / G;
     const long units = H / (group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1);
+    // Steps whose score matrix [Tn, H, ctx] is small (decode rows, short
+    // portions, windows): scores are written once and the heads are mixed
+    // before the values are read, so each value row is read once per key
+    // group. Larger fp32 / odd-size prompt steps apply every head's
+    // weights to every value head and mix afterwards (below).
+    if (path == 1 || (path == 0 && (long)Tn * H * ctx * 4 <= (256L << 20))) {
+        long splits = 8192 / std::max<long>(1, (long)Tn * units);
+        splits = std::min<long>({splits, 32, (ctx + 63) / 64});
+        splits = std::max<long>(splits, 1);
+        Tensor scores = torch::empty({Tn, H, ctx}, f32opt);
+        Tensor part_ml = torch::empty({splits, Tn, H, 2}, f32opt);
+        Tensor part_o;
+        float* po = nullptr;
+        if (splits > 1) {
+            part_o = torch::empty({splits, Tn, H, Dv}, f32opt);
+            po = part_o.data_ptr<float>();
+        }
+        const int rc = launch_talk_attn_scored(
+            q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+            block_table.data_ptr<int>(), (int)block_table.size(1),
+            positions.data_ptr<int>(), seq_idx.data_ptr<int>(),
+            talk.data_ptr<float>(), gate.data_ptr(), gate.stride(0),
+            out.data_ptr(), out.stride(0), scores.data_ptr<float>(), ctx,
+            part_ml.data_ptr<float>(), po, (int)splits, Tn, H, G, D, Dv, bs,
+            (int)window, c, stream());
+        TORCH_CHECK(rc == 0, "talk_attn: head sizes must be <= 256");
+        return;
+    }
     const long nv = G >= 4 ? 4 : G >= 2 ? 2 : 1;
     const long waves = (long)Tn * units * ((G + nv - 1) / nv);
     long splits = 8192 / std::max<long>(1, waves);

@@ -70,7 +70,8 @@ def test_rope_unit_store(dtype, H, G, D, Dv, dims):
         torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
 
 
-def _attn_case(dtype, lens, starts, H, G, D, Dv, window, bs, seed=0):
+def _attn_case(dtype, lens, starts, H, G, D, Dv, window, bs, seed=0,
+               path="auto"):
     torch.manual_seed(seed)
     need = sum(-(-(s + L) // bs) for L, s in zip(lens, starts))
     m = batch_meta(lens, starts, bs, need + 3, seed)
@@ -86,7 +87,7 @@ def _attn_case(dtype, lens, starts, H, G, D, Dv, window, bs, seed=0):
     o2 = torch.zeros_like(o1)
     mq = max(lens)
     ops.talk_attn(q, kc, vc, m["bt"], m["pos"], m["seq"], m["cu"], talk, gate,
-                  window, o1, mq)
+                  window, o1, mq, path)
     ref.talk_attn(q.float(), kc.float(), vc.float(), m["bt"], m["pos"],
                   m["seq"], m["cu"], talk, gate.float(), window, o2)
     return o1.float(), o2.float()
@@ -96,22 +97,27 @@ def _attn_case(dtype, lens, starts, H, G, D, Dv, window, bs, seed=0):
 @pytest.mark.parametrize("H,G,D,Dv,window", [
     (8, 2, 56, 72, 90), (6, 3, 40, 24, 0), (4, 4, 72, 130, 7),
     (5, 1, 33, 17, 20), (16, 8, 64, 64, 50), (12, 6, 16, 200, 1)])
-def test_talk_attn_generic(dtype, H, G, D, Dv, window):
+@pytest.mark.parametrize("path", ["scored", "cross"])
+def test_talk_attn_generic(dtype, H, G, D, Dv, window, path):
     """prompt portions, single rows and a row far into its sequence in one
-    step; pages scattered; windows smaller and larger than the history"""
+    step; pages scattered; windows smaller and larger than the history;
+    both generic forms (heads mixed before / after the values)"""
     a, b = _attn_case(dtype, [5, 1, 33, 1, 2], [0, 120, 17, 0, 300], H, G, D,
-                      Dv, window, 16)
+                      Dv, window, 16, path=path)
     t = tol(dtype)
     torch.testing.assert_close(a, b, rtol=t["rtol"], atol=t["atol"] * 3)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_talk_attn_decode_splits(dtype):
+@pytest.mark.parametrize("path", ["scored", "cross"])
+def test_talk_attn_decode_splits(dtype, path):
     """few rows with long histories: the keys are split over waves"""
-    a, b = _attn_case(dtype, [1, 1, 1], [700, 64, 1300], 8, 2, 64, 64, 0, 64)
+    a, b = _attn_case(dtype, [1, 1, 1], [700, 64, 1300], 8, 2, 64, 64, 0, 64,
+                      path=path)
     t = tol(dtype)
     torch.testing.assert_close(a, b, rtol=t["rtol"], atol=t["atol"] * 3)
-    a, b = _attn_case(dtype, [1, 1], [700, 2000], 8, 4, 128, 128, 512, 256)
+    a, b = _attn_case(dtype, [1, 1], [700, 2000], 8, 4, 128, 128, 512, 256,
+                      path=path)
     torch.testing.assert_close(a, b, rtol=t["rtol"], atol=t["atol"] * 3)
 
 
