@@ -491,7 +491,7 @@ extern "C" int launch_attn_prefill_paged_sink(
 // mixed across heads afterwards: every query head's weights (bf16 hi+lo
 // pair) are applied to the values of ALL key/value heads, so the mix can
 // be taken on the per-(query head, value head) sums:
-//   part[t, h, n, :] = sum_j softmax_h(j) v_n(j)      (normalized, fp32).
+//   part[t, n, h, :] = sum_j softmax_h(j) v_n(j)      (normalized, fp32).
 // Scores use head h's own key head. window > 0: row at absolute position p
 // sees keys p - window < j <= p; key tiles wholly before the tile's first
 // window are skipped. Same tiling and fragment maps as attn_prefill_mfma;
@@ -565,6 +565,29 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
     if (window > 0) kb0 = max(0, hist + q0 - window + 1) / PF_TN * PF_TN;
     constexpr int THREADS_PER_ROW = HD / 8;
 
+    // V^T tile [HD][64 keys] of value head vh. The lanes of a wave take 64
+    // different keys and the same 8 coordinates: the 2-byte transposing
+    // writes of a wave then fall into 32 different LDS banks (with
+    // coordinate-fastest lanes every lane of a key hits the same bank,
+    // because a row pitch that keeps 16-byte reads aligned is a multiple of
+    // the bank count in words).
+    auto stage_vt = [&](int vh, int kb) {
+        for (int i = tid; i < PF_TN * THREADS_PER_ROW; i += 256) {
+            const int key = i % PF_TN;
+            const int d = (i / PF_TN) * 8;
+            const int gk = kb + key;
+            bf16x8 vraw{};
+            if (gk < kv_end) {
+                const long base = (long)bt[gk / bs] * nkv * bs + gk % bs;
+                vraw = load_kv8_bf16(v + (base + (long)vh * bs) * HD + d);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                vt_s[(d + e) * VT_STRIDE + key] =
+                    ((const unsigned short*)&vraw)[e];
+        }
+    };
+
     for (int kb = kb0; kb < kv_end; kb += PF_TN) {
         // ---- stage K tile [64][HD] (own key head) and V^T of value head vh0
         __syncthreads();
@@ -572,18 +595,14 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
             const int key = i / THREADS_PER_ROW;
             const int d = (i % THREADS_PER_ROW) * 8;
             const int gk = kb + key;
-            bf16x8 kraw{}, vraw{};
+            bf16x8 kraw{};
             if (gk < kv_end) {
                 const long base = (long)bt[gk / bs] * nkv * bs + gk % bs;
                 kraw = load_kv8_bf16(k + (base + (long)kvh * bs) * HD + d);
-                vraw = load_kv8_bf16(v + (base + (long)vh0 * bs) * HD + d);
             }
             *reinterpret_cast<bf16x8*>(k_s + key * (HD + PF_PAD) + d) = kraw;
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                vt_s[(d + e) * VT_STRIDE + key] =
-                    ((const unsigned short*)&vraw)[e];
         }
+        stage_vt(vh0, kb);
         __syncthreads();
 
         f32x4 sfrag[PF_TN / 16];
@@ -674,22 +693,7 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
             if (n > 0) {
                 // every wave is done with the previous value head's tile
                 __syncthreads();
-                for (int i = tid; i < PF_TN * THREADS_PER_ROW; i += 256) {
-                    const int key = i / THREADS_PER_ROW;
-                    const int d = (i % THREADS_PER_ROW) * 8;
-                    const int gk = kb + key;
-                    bf16x8 vraw{};
-                    if (gk < kv_end) {
-                        const long base =
-                            (long)bt[gk / bs] * nkv * bs + gk % bs;
-                        vraw = load_kv8_bf16(
-                            v + (base + (long)(vh0 + n) * bs) * HD + d);
-                    }
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        vt_s[(d + e) * VT_STRIDE + key] =
-                            ((const unsigned short*)&vraw)[e];
-                }
+                stage_vt(vh0 + n, kb);
                 __syncthreads();
             }
 #pragma unroll
@@ -717,7 +721,7 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
         for (int n = 0; n < NV; ++n) {
             if (vh0 + n >= nkv) break;
             float* orow =
-                part + (((long)(s0 + qrow) * nq + h) * nkv + vh0 + n) * HD;
+                part + (((long)(s0 + qrow) * nkv + vh0 + n) * nq + h) * HD;
 #pragma unroll
             for (int nb = 0; nb < HD / 16; ++nb)
                 orow[nb * 16 + li] = o_acc[n][nb][r] * inv;
@@ -726,7 +730,7 @@ __global__ __launch_bounds__(256) void attn_prefill_cross_mfma(
 }
 
 // Packed bf16 query chunks against the paged history, each query head's
-// softmax weights applied to every value head: part [T, nq, nkv, hd] fp32.
+// softmax weights applied to every value head: part [T, nkv, nq, hd] fp32.
 // Head size 64 or 128 (returns nonzero otherwise); every score multiplier
 // is already in q.
 extern "C" int launch_attn_prefill_paged_cross(

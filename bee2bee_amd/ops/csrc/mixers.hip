@@ -1455,7 +1455,7 @@ extern "C" int launch_sink_attn(const void* q, long q_tok,
 // Kernel 1 keeps sink_attn's wave layout: one wave per (token, REP query
 // heads of one key group, block of NV value heads, key split); lane = key
 // for the scores, lane = coordinate pair for the value sums. Partials:
-// part_acc [S, T, H, G, Dv] (unnormalized), part_ml [S, T, H, 2].
+// part_acc [S, T, G, H, Dv] (unnormalized), part_ml [S, T, H, 2].
 namespace {
 
 template <typename T, int DPL, int REP, int NV, bool PAIR>
@@ -1577,7 +1577,8 @@ talk_attn_kernel(const T* __restrict__ q, long q_tok,
             for (int i = 0; i < DPL; ++i) {
                 const int d = sa_coord<PAIR>(lane, i);
                 if (d < Dv)
-                    part_acc[(prow * G + v0 + n) * Dv + d] = acc[n][r][i];
+                    part_acc[((((long)split * Tn + t) * G + v0 + n) * H + h) *
+                                 Dv + d] = acc[n][r][i];
             }
         }
     }
@@ -1630,7 +1631,7 @@ talk_mix_kernel(const float* __restrict__ part_acc,
         float a = 0.f;
         for (int s = 0; s < splits; ++s)
             a += wts[s * H + gq] *
-                 part_acc[((((long)s * Tn + t) * H + gq) * G + c) * Dv + d];
+                 part_acc[((((long)s * Tn + t) * G + c) * H + gq) * Dv + d];
         A[idx] = a;
     }
     __syncthreads();

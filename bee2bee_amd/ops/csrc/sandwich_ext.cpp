@@ -249,7 +249,7 @@ void talk_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
         Tensor seq_lens =
             (positions.index_select(0, last.clamp_min(0)) + 1)
                 .to(torch::kInt32);
-        Tensor part = torch::empty({1, Tn, H, G, Dv}, f32opt);
+        Tensor part = torch::empty({1, Tn, G, H, Dv}, f32opt);
         int rc = launch_attn_prefill_paged_cross(
             (const unsigned short*)q.data_ptr(), q.stride(0),
             (const unsigned short*)k_cache.data_ptr(),
@@ -307,7 +307,7 @@ void talk_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
     long splits = 8192 / std::max<long>(1, waves);
     splits = std::min<long>({splits, 32, (ctx + 63) / 64});
     splits = std::max<long>(splits, 1);
-    Tensor part_acc = torch::empty({splits, Tn, H, G, Dv}, f32opt);
+    Tensor part_acc = torch::empty({splits, Tn, G, H, Dv}, f32opt);
     Tensor part_ml = torch::empty({splits, Tn, H, 2}, f32opt);
     int rc = launch_talk_attn(
         q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
