@@ -747,6 +747,10 @@ extern "C" int launch_attn_prefill_paged_cross(
     hipLaunchKernelGGL((attn_prefill_cross_mfma<HDV, NVV>), grid, dim3(256),   \
                        smem, stream, q, k_cache, v_cache, cu, block_table,     \
                        seq_lens, part, nq, nkv, vh0, s_q, W, bs, window)
+    // up to four value heads per launch (measured: two launches of two,
+    // at twice the waves per SIMD, are slower — the scores are recomputed;
+    // so is passing the tiles through registers to prefetch the next one —
+    // the extra registers cost the two-value-head form a wave per SIMD)
     const int nv = nkv > 2 ? 4 : nkv;
     for (int vh0 = 0; vh0 < nkv; vh0 += nv) {
         if (hd == 128) {

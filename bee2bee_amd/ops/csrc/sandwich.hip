@@ -154,8 +154,8 @@ __global__ void add_group_rmsnorm_kernel(float* __restrict__ resid,
 }
 
 // --------------------------------- rotation, unit norm, key/value page store
-// Workgroup per token, a wave per head in turn: H query heads, G key heads,
-// G value heads. Query: q <- unit(rotate(q)) * q_mult in place. Key:
+// Workgroup per (token, four heads), a wave per head: H query heads, G key
+// heads, G value heads. Query: q <- unit(rotate(q)) * q_mult in place. Key:
 // unit(rotate(k)) -> k_cache [n_blocks, G, bs, D]. Value: v -> v_cache
 // [n_blocks, G, bs, Dv]. The rotation pairs coordinate i with i + dims/2
 // over the first `dims` coordinates (cos/sin fp32 tables [max_pos, dims/2],
@@ -181,50 +181,51 @@ rope_unit_store_kernel(T* __restrict__ q, long q_tok, int H,
     const int slot = slot_mapping[t];
     const long blk = slot / bs, off = slot % bs;
     float* nb = buf[wid];
-    for (int hh = wid; hh < H + 2 * G; hh += 4) {
-        if (hh >= H + G) {          // value head: plain copy into its page
-            const int g = hh - H - G;
-            const T* src = v + t * v_tok + (long)g * Dv;
-            T* dst = v_cache + ((blk * G + g) * bs + off) * Dv;
-            for (int i = lane; i < Dv; i += WAVE) dst[i] = src[i];
-            continue;
-        }
-        const bool is_q = hh < H;
-        const int g = hh - H;
-        const T* src = is_q ? q + t * q_tok + (long)hh * D
-                            : k + t * k_tok + (long)g * D;
-        for (int i = lane; i < D; i += WAVE) nb[i] = ldf(src + i);
-        WAVE_LDS_SYNC();
-        // rotated coordinates of this lane (D <= RU_MAXD: at most 8 each)
-        float yv[RU_MAXD / WAVE];
-        float ss = 0.f;
+    // one head per wave: blockIdx.y walks the H + 2G heads four at a time
+    // (no workgroup barrier below, so waves past the end just leave)
+    const int hh = blockIdx.y * 4 + wid;
+    if (hh >= H + 2 * G) return;
+    if (hh >= H + G) {              // value head: plain copy into its page
+        const int g = hh - H - G;
+        const T* src = v + t * v_tok + (long)g * Dv;
+        T* dst = v_cache + ((blk * G + g) * bs + off) * Dv;
+        for (int i = lane; i < Dv; i += WAVE) dst[i] = src[i];
+        return;
+    }
+    const bool is_q = hh < H;
+    const int g = hh - H;
+    const T* src = is_q ? q + t * q_tok + (long)hh * D
+                        : k + t * k_tok + (long)g * D;
+    for (int i = lane; i < D; i += WAVE) nb[i] = ldf(src + i);
+    WAVE_LDS_SYNC();
+    // rotated coordinates of this lane (D <= RU_MAXD: at most 8 each)
+    float yv[RU_MAXD / WAVE];
+    float ss = 0.f;
 #pragma unroll
-        for (int c = 0; c < RU_MAXD / WAVE; ++c) {
-            const int i = lane + c * WAVE;
-            float y = 0.f;
-            if (i < D) {
-                y = nb[i];
-                if (i < dims) {
-                    const int j = i < half ? i : i - half;
-                    const float yp = nb[i < half ? i + half : i - half];
-                    const float cs = cos_t[(long)pos * half + j];
-                    const float sn = sin_t[(long)pos * half + j];
-                    y = i < half ? y * cs - yp * sn : y * cs + yp * sn;
-                }
+    for (int c = 0; c < RU_MAXD / WAVE; ++c) {
+        const int i = lane + c * WAVE;
+        float y = 0.f;
+        if (i < D) {
+            y = nb[i];
+            if (i < dims) {
+                const int j = i < half ? i : i - half;
+                const float yp = nb[i < half ? i + half : i - half];
+                const float cs = cos_t[(long)pos * half + j];
+                const float sn = sin_t[(long)pos * half + j];
+                y = i < half ? y * cs - yp * sn : y * cs + yp * sn;
             }
-            yv[c] = y;
-            ss += y * y;
         }
-        const float r = 1.f / sqrtf(wave_sum(ss) / (float)D + eps) *
-                        (is_q ? q_mult : 1.f);
-        T* dst = is_q ? q + t * q_tok + (long)hh * D
-                      : k_cache + ((blk * G + g) * bs + off) * D;
+        yv[c] = y;
+        ss += y * y;
+    }
+    const float r = 1.f / sqrtf(wave_sum(ss) / (float)D + eps) *
+                    (is_q ? q_mult : 1.f);
+    T* dst = is_q ? q + t * q_tok + (long)hh * D
+                  : k_cache + ((blk * G + g) * bs + off) * D;
 #pragma unroll
-        for (int c = 0; c < RU_MAXD / WAVE; ++c) {
-            const int i = lane + c * WAVE;
-            if (i < D) stf(dst + i, yv[c] * r);
-        }
-        WAVE_LDS_SYNC();
+    for (int c = 0; c < RU_MAXD / WAVE; ++c) {
+        const int i = lane + c * WAVE;
+        if (i < D) stf(dst + i, yv[c] * r);
     }
 }
 
@@ -340,13 +341,14 @@ extern "C" int launch_rope_unit_store(
     const int* slot_mapping, long T, int f32, hipStream_t s) {
     if (D > RU_MAXD) return 1;
     if (T == 0) return 0;
+    const dim3 grid(T, (H + 2 * G + 3) / 4);
     if (f32)
-        rope_unit_store_kernel<float><<<T, 256, 0, s>>>(
+        rope_unit_store_kernel<float><<<grid, 256, 0, s>>>(
             (float*)q, q_tok, H, (const float*)k, k_tok, (const float*)v,
             v_tok, G, D, Dv, eps, dims, positions, cos_t, sin_t, q_mult,
             (float*)k_cache, (float*)v_cache, bs, slot_mapping);
     else
-        rope_unit_store_kernel<unsigned short><<<T, 256, 0, s>>>(
+        rope_unit_store_kernel<unsigned short><<<grid, 256, 0, s>>>(
             (unsigned short*)q, q_tok, H, (const unsigned short*)k, k_tok,
             (const unsigned short*)v, v_tok, G, D, Dv, eps, dims, positions,
             cos_t, sin_t, q_mult, (unsigned short*)k_cache,
