@@ -526,3 +526,23 @@ def test_random_init_runs_and_is_consistent():
     whole = replay(eng, {"a": toks}, [[("a", 20)]])["a"]
     steps = replay(eng, {"a": toks}, [[("a", 1)]] * 20)["a"]
     assert rel_err(steps, whole) < 1e-4
+
+
+def test_bench_compare_option_runs_on_cpu():
+    """bench.py --compare-pimodra: one JSON line per model with prefill and
+    decode throughput (CPU run: small stand-in sizes)."""
+    import os
+    import subprocess
+
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run(
+        [sys.executable, os.path.join(repo, "bench.py"), "--compare-pimodra",
+         "s", "--steps", "1", "--warmup", "0"],
+        capture_output=True, text=True, timeout=300,
+        env=dict(os.environ, HIP_VISIBLE_DEVICES="", CUDA_VISIBLE_DEVICES=""))
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [json.loads(x) for x in r.stdout.splitlines() if x.startswith("{")]
+    assert [x["model"] for x in lines] == ["pimodra-s", "gqa-moe-s"]
+    for x in lines:
+        assert x["compare"] == "pimodra-vs-dense"
+        assert x["prefill_tokens_per_s"] > 0 and x["decode_tokens_per_s"] > 0
