@@ -23,8 +23,11 @@ the SAME page and slot bookkeeping:
   * every layer with a convolution: the last taps-1 conv inputs
     [n_slots, taps-1, channels] per sequence slot (the mixer input for the
     whole-width conv, the q|k|v projection for a delta mixer's short conv);
-  * a parallel mixer (attention + delta rule side by side) has pages AND
-    state in the same layer.
+  * grouped-query attention with a short convolution on its projected
+    q|k|v: the two page pools and the last taps-1 projected rows per slot;
+  * an element-wise gated recurrence (minGRU): state [n_slots, width] fp32;
+  * a parallel mixer (attention + delta rule or minGRU side by side) has
+    pages AND state in the same layer.
 A sequence owns one state slot from new_seq to free_seq. Slots and pages
 are handed out again without clearing: the kernels never read state or
 cache rows that precede a sequence's position 0.
@@ -110,7 +113,8 @@ class PagedKV:
                 if m.kind == "latent_attention":
                     k = torch.zeros(self.n_blocks, self.block_size,
                                     m.cache_dim, device=dev, dtype=self.dtype)
-                elif m.kind in ("sink_attention", "talk_attention"):
+                elif m.kind in ("sink_attention", "talk_attention",
+                                "gqa_attention"):
                     # the dense models' page layout: one (key, head) row
                     # contiguous; values here are the raw key projection
                     k = torch.zeros(self.n_blocks, m.kv_heads,
@@ -119,6 +123,14 @@ class PagedKV:
                     v = torch.zeros(self.n_blocks, m.kv_heads,
                                     self.block_size, m.vdim, device=dev,
                                     dtype=self.dtype)
+                    if m.kind == "gqa_attention" and m.taps > 1:
+                        # the last taps-1 projected q|k|v rows
+                        conv = torch.zeros(n_slots, m.taps - 1,
+                                           m.conv_channels, device=dev,
+                                           dtype=self.dtype)
+                elif m.kind == "min_gru":
+                    rec = torch.zeros(n_slots, m.width, device=dev,
+                                      dtype=f32)
                 else:   # lightning / retention / delta: recurrent state
                     rec = torch.zeros(n_slots, m.heads, m.dim, m.vdim,
                                       device=dev, dtype=f32)

@@ -223,10 +223,14 @@ class Runner:
             def act_fn(gu):
                 if ffn.act == "silu_glu":
                     return ops.silu_glu(gu)
+                if ffn.act == "gelu":
+                    return ops.gelu_erf(gu)
                 return ops.clamped_glu(gu, ffn.limit, ffn.alpha)
         else:
             E, I, top_k = s.n_experts, s.intermediate_size, s.top_k_experts
             act_fn = ops.swiglu
+        # rows of an expert's input-side matrix: gate|up, or up alone
+        U = lw.moe_w_gate_up.shape[1]
         if ffn is None and self.ep is not None:
             if self.weights.expert_range is not None:
                 # weights hold only this rank's expert shard (EP sharding)
@@ -238,10 +242,12 @@ class Runner:
             return self.ep.forward(x, lw.moe_gate, w_gu, w_dn)
         if ffn is None:
             logits = F.linear(x, lw.moe_gate)
-        if ffn is not None and ffn.score == "softmax_all":
+        if ffn is not None and ffn.score in ("softmax_all", "sigmoid_all"):
             # scores over all experts, group-limited choice, no renorm
-            weights, idx = ops.group_topk_gate(logits, top_k, ffn.n_groups,
-                                               ffn.keep_groups)
+            weights, idx = ops.group_topk_gate(
+                logits, top_k, ffn.n_groups, ffn.keep_groups,
+                "sigmoid" if ffn.score == "sigmoid_all" else "softmax",
+                ffn.group_top)
         else:
             weights, idx = ops.moe_topk_gate(logits, top_k)  # [T,k]
         T, H = x.shape
@@ -249,7 +255,7 @@ class Runner:
         if T <= self.MOE_DENSE_MAX_TOKENS:
             x_e = x.unsqueeze(0).expand(E, T, H)
             gu = torch.bmm(x_e, lw.moe_w_gate_up.transpose(1, 2))  # [E,T,2I]
-            act = act_fn(gu.reshape(E * T, 2 * I)).view(E, T, I)
+            act = act_fn(gu.reshape(E * T, U)).view(E, T, I)
             y = torch.bmm(act, lw.moe_w_down.transpose(1, 2))  # [E,T,H]
             wfull = torch.zeros(T, E, dtype=torch.float32, device=x.device)
             wfull.scatter_(1, idx.long(), weights)
@@ -308,7 +314,7 @@ class Runner:
                 padded = torch.zeros(E, C, H, dtype=x.dtype, device=x.device)
                 padded[flat_e, rank] = x[tok]
                 gu = torch.bmm(padded, lw.moe_w_gate_up.transpose(1, 2))
-                act = act_fn(gu.reshape(E * C, 2 * I)).view(E, C, I)
+                act = act_fn(gu.reshape(E * C, U)).view(E, C, I)
                 y = torch.bmm(act, lw.moe_w_down.transpose(1, 2))  # [E,C,H]
                 contrib = y[flat_e, rank].float()  # [S, H] slot order
             out = torch.zeros(T, H, dtype=torch.float32, device=x.device)
@@ -433,7 +439,11 @@ class Runner:
                tuple(sorted(scaling.items())) if scaling else None)
         t = self._rope_by_cfg.get(key)
         if t is None:
-            if scaling:
+            if scaling and "kind" in scaling:
+                # linear or banded frequency scaling
+                t = ops.rope_freq_tables(self.spec.max_seq_len, dims, base,
+                                         scaling, self.device)
+            elif scaling:
                 t = ops.rope_tables_scaled(self.spec.max_seq_len, dims, base,
                                            scaling, self.device)
             else:
@@ -478,6 +488,8 @@ class Runner:
         n = s.n_layers
         if s.layer_specs[0].form == "sandwich_w":
             return self._forward_sandwich_w(x, meta)
+        if s.layer_specs[0].form == "parallel_gated":
+            return self._forward_parallel_gated(x, meta)
         if s.layer_specs[0].form == "parallel":
             # x += mixer(h) + ffn(h), h = unit(x) * w: the residual add and
             # the next layer's norm run as one kernel
@@ -636,6 +648,162 @@ class Runner:
         ops.talk_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
                       cu, lw.talk, gate, m.window, out, max_qlen)
         return F.linear(out, lw.wo)
+
+    # ------------------------------------------ gated parallel-form layers
+
+    def _forward_parallel_gated(self, x: torch.Tensor, meta) -> torch.Tensor:
+        """x += sigmoid(g1) * mixer(h) + sigmoid(g2) * ffn(h) with h =
+        unit(x) * w and both gates projections of h. The layer list is the
+        list of RUNS (a repeated block appears once per pass, sharing
+        weights but not pages or state); a run with `readd_embed` adds the
+        embedding output to the residual first. The two gated adds, that
+        add and the next run's norm are ONE kernel."""
+        s, W = self.spec, self.weights
+        eps, dt, n = s.rms_eps, self.dtype, s.n_layers
+        e0 = x.clone() if any(l.readd_embed for l in s.layer_specs) else None
+        normed = ops.rmsnorm_f32(x, W.layers[0].norm_w, eps, dt)
+        for i in range(n):
+            y1, g1, y2, g2 = self._gated_layer(i, normed, meta)
+            nxt = W.layers[i + 1].norm_w if i + 1 < n else None
+            extra = e0 if i + 1 < n and s.layer_specs[i + 1].readd_embed \
+                else None
+            if self.layer_tap is not None and extra is not None:
+                # the probe sees the residual before the next pass's add
+                ops.gated_add_rmsnorm(x, y1, g1, y2, g2, None, None, eps, dt)
+                self.layer_tap(i, x)
+                normed = ops.gated_add_rmsnorm(x, None, None, None, None,
+                                               extra, nxt, eps, dt)
+                continue
+            normed = ops.gated_add_rmsnorm(x, y1, g1, y2, g2, extra, nxt,
+                                           eps, dt)
+            if self.layer_tap is not None:
+                self.layer_tap(i, x)
+        return x
+
+    def _gated_layer(self, i: int, h: torch.Tensor, meta):
+        """Sublayer outputs and raw gates of layer run i: (mixer(h), g1,
+        ffn(h) or None, g2 or None). One input GEMM (with its bias vector)
+        covers every projection that reads h, the gates included."""
+        from ..models.hybrid import mixer_parts
+
+        s = self.spec
+        lw, l = self.weights.layers[i], s.layer_specs[i]
+        ins, _ = lw.layout
+        proj = F.linear(h, lw.w_in, lw.b_in)
+
+        def cols(key):
+            off, n = ins[key]
+            return proj[:, off : off + n]
+
+        m = l.mixer
+        ys = []
+        for pre, part in mixer_parts(m):
+            ns = lw.mix[pre]
+            if part.kind == "gqa_attention":
+                o = self._gqa_attn_part(i, part, ns, cols, pre, meta)
+            elif part.kind == "latent_attention":
+                o = self._latent_attn_part(i, part, ns, cols, pre, meta)
+            else:
+                o = self._min_gru_part(i, part, cols, pre, meta)
+            ys.append(F.linear(o, ns.wo, ns.wo_b))
+        if m.kind == "parallel":
+            if m.combine != "normed_mean":
+                raise ValueError(f"unknown combine {m.combine!r}")
+            y1 = ops.pair_rmsnorm_mean(
+                ys[0], lw.mix["left."].out_norm, ys[1],
+                lw.mix["right."].out_norm, s.rms_eps, self.dtype)
+        else:
+            y1 = ys[0]
+        if l.ffn is None:
+            return y1, cols("rg1"), None, None
+        y2 = self._moe_mlp(lw, h, ffn=l.ffn)
+        return y1, cols("rg1"), y2, cols("rg2")
+
+    def _gqa_attn_part(self, i: int, m, ns, cols, pre, meta) -> torch.Tensor:
+        """Grouped-query attention of layer run i: optional short conv on
+        the projected q|k|v (fp32 out), rotation + page store, attention
+        with the spec's cap / score mix / sink / window / head gate."""
+        (positions, slot_mapping, cu, seq_idx, block_table, state_slots,
+         max_qlen) = meta
+        T = positions.shape[0]
+        nq, nk, nv = m.heads * m.dim, m.kv_heads * m.dim, m.kv_heads * m.vdim
+        off = cols(pre + "q")
+        qkv = off.as_strided((T, nq + nk + nv), off.stride())
+        if ns.conv_w is not None:
+            qkv = ops.short_conv(qkv, ns.conv_w, self.kv.conv_state[i],
+                                 state_slots, cu, seq_idx, positions, False)
+        q = qkv[:, :nq].view(T, m.heads, m.dim)
+        k = qkv[:, nq : nq + nk].view(T, m.kv_heads, m.dim)
+        v = qkv[:, nq + nk :].view(T, m.kv_heads, m.vdim)
+        cos = sin = None
+        if m.rope_dims:
+            cos, sin = self._rope_tables(m.rope_dims, m.rope_base, f64=True,
+                                         scaling=m.rope_scaling)
+        k_cache, v_cache = self.kv.k_cache[i], self.kv.v_cache[i]
+        # the query leaves this rotated and times the score scale
+        if q.dtype == self.dtype:
+            q_out = q
+        else:
+            q_out = torch.empty(T, m.heads, m.dim, dtype=self.dtype,
+                                device=q.device)
+        ops.rope_store(q, k, v, q_out, m.rope_dims,
+                       m.rope_layout == "interleaved", positions, cos, sin,
+                       m.scale, k_cache, v_cache, slot_mapping)
+        sink = None
+        if m.zero_sink:
+            sink = self._zeros_f32(m.heads)
+        out = torch.empty(T, m.out_size, dtype=self.dtype, device=q.device)
+        ops.gqa_attn(q_out, k_cache, v_cache, block_table, positions, seq_idx,
+                     cu, m.softcap, ns.talk if m.score_mix else None, sink,
+                     cols(pre + "g") if m.head_gate else None, m.window, out,
+                     max_qlen)
+        return out
+
+    def _zeros_f32(self, n: int) -> torch.Tensor:
+        z = self._rope_by_cfg.get(("zeros", n))
+        if z is None:
+            z = self._rope_by_cfg[("zeros", n)] = torch.zeros(
+                n, dtype=torch.float32, device=self.device)
+        return z
+
+    def _latent_attn_part(self, i: int, m, ns, cols, pre, meta
+                          ) -> torch.Tensor:
+        """Latent attention of layer run i in absorbed form (the key
+        up-projection folded into the query, the value up-projection into
+        the output), queries through their own normed latent when the spec
+        has one, a per-head sink and sigmoid head gate in the kernel."""
+        (positions, slot_mapping, cu, seq_idx, block_table, _,
+         max_qlen) = meta
+        T, H = positions.shape[0], m.heads
+        D, R, C = m.dim, m.rot_dim, m.kv_rank
+        if m.q_rank:
+            cq = ops.slice_rmsnorm(cols(pre + "dq"), ns.q_norm,
+                                   self.spec.rms_eps)
+            q = F.linear(cq, ns.w_uq).view(T, H, D + R)
+        else:
+            q = cols(pre + "q").view(T, H, D + R)
+        kv, gate = cols(pre + "dkv"), cols(pre + "g")
+        cache = self.kv.k_cache[i]
+        cos, sin = self._rope_tables(m.rope_dims, m.rope_base, f64=True)
+        ops.latent_rope_store(q[..., D:], kv, ns.kv_norm, self.spec.rms_eps,
+                              C, m.rope_dims, positions, cos, sin, cache,
+                              slot_mapping)
+        q_abs = torch.bmm(q[..., :D].transpose(0, 1), ns.w_uk)    # [H,T,C]
+        lat = ops.latent_attn(q_abs, q[..., D:], gate, cache, block_table,
+                              positions, seq_idx, cu, m.window, m.scale,
+                              max_qlen, sink=ns.sink)
+        o = torch.bmm(lat, ns.w_uv)                              # [H,T,Dv]
+        return o.transpose(0, 1).reshape(T, H * m.vdim)
+
+    def _min_gru_part(self, i: int, m, cols, pre, meta) -> torch.Tensor:
+        positions, _, cu, _, _, state_slots, max_qlen = meta
+        T = positions.shape[0]
+        out = torch.empty(T, m.width, dtype=self.dtype,
+                          device=positions.device)
+        ops.min_gru(cols(pre + "z"), cols(pre + "x"), cols(pre + "g"),
+                    self.kv.rec_state[i], state_slots, cu, positions, out,
+                    max_qlen)
+        return out
 
     # ------------------------------------------------- parallel-form layers
 

@@ -32,6 +32,21 @@ sublayer; a block of layers may run several times with the same tensors):
   rot.{base, dims, scaling.{factor, original, fast, slow}}},
   layers[i].mlp.{kind: dense, ff} | {kind: moe, expert.ff,
   router.{experts, top, groups.{count, keep}}} (or null).
+
+Zevilorn config.json keys (parallel-form layers whose two sublayer outputs
+each pass a sigmoid gate computed from the normed input; a block of layers
+may run several times with the same tensors, the embedding output being
+added back before every later pass):
+  architecture, vocab, width, norm.eps, loop.{start, stop, times} (or absent),
+  layers[i].type in {attention, latent_attention, parallel},
+  attention: mixer.{heads, kv_heads, dim, vdim, scale, softcap, conv,
+  mask.size, rot.{base, dims, scaling.{factor, low, high, original}}},
+  latent_attention: mixer.{heads, dim, rot_dim, vdim, kv_rank, q_rank, scale,
+  rot.{base, dims}},
+  parallel: mixer.left.{heads, kv_heads, dim, vdim, scale, mask.size,
+  rot.{base, dims, scaling.{factor}}}, mixer.right.{width},
+  layers[i].mlp.{kind: moe, expert.ff, router.{experts, top,
+  groups.{count, keep}}} (or null).
 """
 from __future__ import annotations
 
@@ -49,12 +64,28 @@ class LatentAttnSpec:
     rot_dim: int        # rotated query/key dims per head
     vdim: int
     kv_rank: int
-    window: int         # query i sees keys j with 0 <= i - j < window
+    window: int         # query i sees keys j with 0 <= i - j < window;
+                        # 0: every earlier position
     rope_base: float
     rope_dims: int      # leading dims of the rot part that rotate
     scale: float
+    # queries through a normed latent of this width (0: one full projection)
+    q_rank: int = 0
+    # a learned logit per head that counts once in the softmax denominator
+    # and has neither key nor value
+    sink: bool = False
 
     kind = "latent_attention"
+
+    @property
+    def in_sizes(self) -> Tuple[Tuple[str, int], ...]:
+        """Rows of the fused input projection, in order."""
+        return (("dq" if self.q_rank else "q", self.q_rank or self.q_size),
+                ("dkv", self.cache_dim), ("g", self.heads))
+
+    @property
+    def out_size(self) -> int:
+        return self.heads * self.vdim
 
     @property
     def q_size(self) -> int:
@@ -210,12 +241,89 @@ class TalkAttnSpec:
 
 
 @dataclass
+class GqaAttnSpec:
+    """Grouped-query softmax attention over paged keys and values whose
+    extras are all options: biases on q/k/v/o, a short causal per-channel
+    convolution on the projected q, k, v (taps > 1; the last taps-1
+    projected rows are carried per sequence), rotation of the first
+    rope_dims coordinates in the interleaved (2i, 2i+1) or half (i, i+n)
+    layout with an optional frequency scaling, a tanh cap on the scaled
+    scores (softcap > 0), a learned heads x heads mix of the capped scores
+    BEFORE the softmax (score_mix), a sliding window (0: none), a
+    zero-logit sink in the softmax denominator (zero_sink: one is added to
+    the sum), and a sigmoid gate per head on the output (head_gate).
+    rope_scaling: None, {"kind": "linear", "factor"} (every frequency
+    divided by factor) or {"kind": "banded", "factor", "low", "high",
+    "original"} (wavelengths above original/low slowed by factor, below
+    original/high kept, a linear blend between)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0
+    rope_base: float = 10000.0
+    rope_dims: int = 0
+    rope_layout: str = "interleaved"
+    rope_scaling: Optional[Dict[str, Any]] = None
+    softcap: float = 0.0
+    score_mix: bool = False
+    zero_sink: bool = False
+    bias: bool = False
+    taps: int = 0
+    head_gate: bool = False
+
+    kind = "gqa_attention"
+
+    @property
+    def conv_channels(self) -> int:
+        return (self.heads + self.kv_heads) * self.dim + \
+            self.kv_heads * self.vdim
+
+    @property
+    def in_sizes(self) -> Tuple[Tuple[str, int], ...]:
+        """Rows of the fused input projection, in order (q, k, v are
+        neighbours so one convolution covers them)."""
+        out = (("q", self.heads * self.dim), ("k", self.kv_heads * self.dim),
+               ("v", self.kv_heads * self.vdim))
+        return out + ((("g", self.heads),) if self.head_gate else ())
+
+    @property
+    def out_size(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclass
+class MinGRUSpec:
+    """Element-wise gated recurrence whose gates read only the current
+    token: z = sigmoid(W_z h + b_z), u = W_x h + b_x, candidate c = u + 1/2
+    (u >= 0) or sigmoid(u) (u < 0), S_t = (1 - z) S_(t-1) + z c, output
+    S_t * silu(W_g h). State [width] fp32 per sequence, zero at the start."""
+    width: int
+
+    kind = "min_gru"
+    heads = 1
+    dim = 1
+
+    @property
+    def in_sizes(self) -> Tuple[Tuple[str, int], ...]:
+        return (("z", self.width), ("x", self.width), ("g", self.width))
+
+    @property
+    def out_size(self) -> int:
+        return self.width
+
+
+@dataclass
 class ParallelMixerSpec:
-    """Two mixers on the same input, summed with fixed scales."""
-    left: Any               # SinkAttnSpec
-    right: Any              # DeltaSpec
-    left_scale: float
-    right_scale: float
+    """Two mixers on the same input. combine "scaled_sum": summed with
+    fixed scales; "normed_mean": each side's projected output is RMS-normed
+    over the model width with a weight of its own, then half their sum."""
+    left: Any               # SinkAttnSpec | GqaAttnSpec
+    right: Any              # DeltaSpec | MinGRUSpec
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    combine: str = "scaled_sum"
 
     kind = "parallel"
 
@@ -248,7 +356,11 @@ class MoEFFNSpec:
     the top-k scores are the weights as they are (no renormalization); with
     n_groups > 1 the experts form equal groups of neighbours, a group's
     score is its largest expert score, and only experts of the best
-    keep_groups groups can be chosen."""
+    keep_groups groups can be chosen. score "sigmoid_all": as "softmax_all"
+    with scores = sigmoid of each logit. group_top: a group's score is the
+    sum of its group_top largest expert scores.
+    act "gelu": experts without a gate, y = down(gelu(up h)), exact (erf)
+    gelu."""
     n_experts: int
     top_k: int
     ff: int
@@ -260,6 +372,12 @@ class MoEFFNSpec:
     score: str = "softmax_topk"
     n_groups: int = 1
     keep_groups: int = 1
+    group_top: int = 1
+
+    @property
+    def up_rows(self) -> int:
+        """Rows of one expert's input-side matrix."""
+        return self.ff if self.act == "gelu" else 2 * self.ff
 
 
 @dataclass
@@ -269,6 +387,8 @@ class LayerSpec:
     # "sandwich": scalar-gain norms before and after each sublayer, mixer
     # then feed-forward. "parallel": x += mixer(h) + ffn(h), h = norm(x) * w.
     # "sandwich_w": as "sandwich" with weighted, grouped RMS norms.
+    # "parallel_gated": x += sigmoid(W1 h + b1) * mixer(h)
+    #                      + sigmoid(W2 h + b2) * ffn(h), h = norm(x) * w.
     form: str = "sandwich"
     # layer whose tensors this layer uses (its own cache and state)
     weights_of: Optional[int] = None
@@ -277,6 +397,9 @@ class LayerSpec:
     step_row: Optional[int] = None
     # index of the checkpoint layer ('l<src>.') this run executes
     src: Optional[int] = None
+    # the embedding output is added to the residual right before this run
+    # (the first layer of every pass but the first over a repeated block)
+    readd_embed: bool = False
 
     @property
     def kind(self) -> str:
@@ -433,6 +556,21 @@ def _pimodra_ffn_from_cfg(f: Optional[Dict[str, Any]]):
                       score="softmax_all", n_groups=n_g, keep_groups=keep)
 
 
+def _loop_order(n: int, loop: Optional[Dict[str, Any]]
+                ) -> List[Tuple[int, Optional[int]]]:
+    """[(checkpoint layer, pass number or None)] in execution order: layers
+    start..stop-1 run `times` times in a row, the rest once."""
+    if not loop:
+        return [(i, None) for i in range(n)]
+    a, b, times = int(loop["start"]), int(loop["stop"]), int(loop["times"])
+    if not (0 <= a < b <= n and times >= 1):
+        raise ValueError("loop: need 0 <= start < stop <= layers, times >= 1")
+    order: List[Tuple[int, Optional[int]]] = [(i, None) for i in range(a)]
+    for t in range(times):
+        order += [(i, t) for i in range(a, b)]
+    return order + [(i, None) for i in range(b, n)]
+
+
 def looped_layer_specs_from_cfg(layers: List[Dict[str, Any]],
                                 loop: Optional[Dict[str, Any]]
                                 ) -> List[LayerSpec]:
@@ -441,16 +579,7 @@ def looped_layer_specs_from_cfg(layers: List[Dict[str, Any]],
     is a LayerSpec of its own (own pages), runs after the first pass name
     the first pass's run as `weights_of`, and the first run of each pass
     carries the pass number as `step_row`."""
-    n = len(layers)
-    order: List[Tuple[int, Optional[int]]] = [(i, None) for i in range(n)]
-    if loop:
-        a, b, times = int(loop["start"]), int(loop["stop"]), int(loop["times"])
-        if not (0 <= a < b <= n and times >= 1):
-            raise ValueError("loop: need 0 <= start < stop <= layers, times >= 1")
-        order = [(i, None) for i in range(a)]
-        for t in range(times):
-            order += [(i, t) for i in range(a, b)]
-        order += [(i, None) for i in range(b, n)]
+    order = _loop_order(len(layers), loop)
     out: List[LayerSpec] = []
     first_run: Dict[int, int] = {}
     for run, (i, t) in enumerate(order):
@@ -465,6 +594,124 @@ def looped_layer_specs_from_cfg(layers: List[Dict[str, Any]],
             step_row=t if (t is not None and i == int(loop["start"])) else None,
             src=i))
     return out
+
+
+def _rot_scaling(sc: Optional[Dict[str, Any]]) -> Optional[Dict[str, Any]]:
+    """A rot.scaling entry: with 'original' the banded rule, with only a
+    factor the linear one."""
+    if not sc:
+        return None
+    if "original" in sc:
+        return {"kind": "banded", "factor": float(sc["factor"]),
+                "low": float(sc["low"]), "high": float(sc["high"]),
+                "original": float(sc["original"])}
+    return {"kind": "linear", "factor": float(sc["factor"])}
+
+
+def _gqa_attn_from_cfg(m: Dict[str, Any], **options: Any) -> GqaAttnSpec:
+    heads = int(m["heads"])
+    kv_heads = int(m.get("kv_heads", heads))
+    if heads % kv_heads:
+        raise ValueError("attention: heads must be a multiple of kv_heads")
+    rot = m.get("rot") or {}
+    dims = int(rot.get("dims", 0))
+    if dims % 2 or dims > int(m["dim"]):
+        raise ValueError("attention: rot.dims must be even and <= dim")
+    return GqaAttnSpec(
+        heads=heads, kv_heads=kv_heads, dim=int(m["dim"]),
+        vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+        window=int((m.get("mask") or {}).get("size", 0) or 0),
+        rope_base=float(rot.get("base", 10000.0)), rope_dims=dims,
+        rope_layout="interleaved",
+        rope_scaling=_rot_scaling(rot.get("scaling")),
+        softcap=float(m.get("softcap") or 0.0),
+        taps=int(m.get("conv") or 0), **options)
+
+
+def _zevilorn_mixer_from_cfg(kind: str, m: Dict[str, Any]):
+    if kind == "attention":
+        return _gqa_attn_from_cfg(m, score_mix=True, zero_sink=True,
+                                  bias=True)
+    if kind == "latent_attention":
+        rot = m.get("rot") or {}
+        rot_dim = int(m["rot_dim"])
+        dims = int(rot.get("dims", rot_dim))
+        if dims % 2 or dims > rot_dim:
+            raise ValueError("latent attention: rot.dims must be even and "
+                             "<= rot_dim")
+        return LatentAttnSpec(
+            heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=rot_dim,
+            vdim=int(m["vdim"]), kv_rank=int(m["kv_rank"]),
+            window=int((m.get("mask") or {}).get("size", 0) or 0),
+            rope_base=float(rot.get("base", 10000.0)), rope_dims=dims,
+            scale=float(m["scale"]), q_rank=int(m.get("q_rank") or 0),
+            sink=True)
+    if kind == "parallel":
+        return ParallelMixerSpec(
+            left=_gqa_attn_from_cfg(m["left"], head_gate=True),
+            right=MinGRUSpec(width=int(m["right"]["width"])),
+            combine="normed_mean")
+    raise ValueError(f"unknown mixer type {kind!r}")
+
+
+def _zevilorn_ffn_from_cfg(f: Optional[Dict[str, Any]]):
+    if not f:
+        return None
+    if f.get("kind", "moe") != "moe":
+        raise ValueError(f"unknown feed-forward kind {f.get('kind')!r}")
+    r = f["router"]
+    g = r.get("groups") or {}
+    E, n_g = int(r["experts"]), int(g.get("count", 1))
+    keep = int(g.get("keep", n_g))
+    if E % n_g or not 1 <= keep <= n_g:
+        raise ValueError("router: experts must split into equal groups")
+    if int(r["top"]) > keep * (E // n_g):
+        raise ValueError("router: top exceeds the experts of the kept groups")
+    return MoEFFNSpec(n_experts=E, top_k=int(r["top"]),
+                      ff=int(f["expert"]["ff"]), act="gelu",
+                      score="sigmoid_all", n_groups=n_g, keep_groups=keep,
+                      group_top=min(2, E // n_g))
+
+
+def gated_layer_specs_from_cfg(layers: List[Dict[str, Any]],
+                               loop: Optional[Dict[str, Any]]
+                               ) -> List[LayerSpec]:
+    """Zevilorn: the list of layer RUNS in execution order (a repeated
+    block appears once per pass; runs after the first pass name the first
+    pass's run as `weights_of` and keep pages and state of their own). The
+    first run of every pass but the first has `readd_embed`."""
+    out: List[LayerSpec] = []
+    first_run: Dict[int, int] = {}
+    for run, (i, t) in enumerate(_loop_order(len(layers), loop)):
+        l = layers[i]
+        owner = first_run.setdefault(i, run)
+        out.append(LayerSpec(
+            mixer=_zevilorn_mixer_from_cfg(l["type"], l["mixer"]),
+            ffn=_zevilorn_ffn_from_cfg(l.get("mlp")), form="parallel_gated",
+            weights_of=None if owner == run else owner, src=i,
+            readd_embed=bool(t and i == int(loop["start"]))))
+    return out
+
+
+def gated_layout(l: LayerSpec, width: int
+                 ) -> Tuple[Dict[str, Tuple[int, int]], int]:
+    """Rows of a gated parallel-form layer's ONE input matrix: every
+    projection that reads the normed h — the mixer's (per part, in in_sizes
+    order), then the two residual gates 'rg1' (mixer) and 'rg2'
+    (feed-forward, when there is one). Every segment starts on a multiple of
+    8 rows. Returns ({name: (offset, size)}, total)."""
+    ins: Dict[str, Tuple[int, int]] = {}
+    a = 0
+    for pre, m in mixer_parts(l.mixer):
+        for name, n in m.in_sizes:
+            ins[pre + name] = (a, n)
+            # q, k, v stay neighbours (one conv / one rotation pass)
+            a += n if name in ("q", "k") and m.kind == "gqa_attention" \
+                else _pad8(n)
+    for name in ("rg1", "rg2") if l.ffn is not None else ("rg1",):
+        ins[name] = (a, width)
+        a += _pad8(width)
+    return ins, a
 
 
 def complete_from_shapes(layers: List[LayerSpec],
@@ -537,6 +784,10 @@ def hybrid_n_params(width: int, vocab: int, taps: int,
             if l.weights_of is None or active_only:
                 n += _sandwich_w_layer_params(width, l, active_only)
             continue
+        if l.form == "parallel_gated":
+            if l.weights_of is None or active_only:
+                n += _gated_layer_params(width, l, active_only)
+            continue
         n += 4 + width * taps
         if m.kind == "latent_attention":
             n += width * (m.q_size + m.cache_dim + m.heads) + m.kv_rank
@@ -561,6 +812,36 @@ def _sandwich_w_layer_params(width: int, l: LayerSpec,
     elif f is not None:
         e = f.top_k if active_only else f.n_experts
         n += 2 * width + width * f.n_experts + 3 * width * e * f.ff
+    return n
+
+
+def _gated_layer_params(width: int, l: LayerSpec, active_only: bool) -> int:
+    n = width + width * (width + 1)                 # norm, mixer gate
+    for _, m in mixer_parts(l.mixer):
+        n += width * m.out_size
+        if m.kind == "latent_attention":
+            n += width * (m.cache_dim + m.heads) + m.kv_rank + m.heads
+            n += m.kv_rank * m.heads * (m.dim + m.vdim)
+            n += (m.q_rank * (width + 1 + m.q_size) if m.q_rank
+                  else width * m.q_size)
+        elif m.kind == "gqa_attention":
+            rows = sum(sz for _, sz in m.in_sizes)
+            n += width * rows
+            if m.bias:
+                n += m.conv_channels + width
+            if m.taps > 1:
+                n += m.taps * m.conv_channels
+            if m.score_mix:
+                n += m.heads * m.heads
+        else:
+            n += 3 * width * m.width + 2 * m.width
+    if l.mixer.kind == "parallel" and l.mixer.combine == "normed_mean":
+        n += 2 * width
+    f = l.ffn
+    if f is not None:
+        e = f.top_k if active_only else f.n_experts
+        n += width * (width + 1) + width * f.n_experts
+        n += e * f.ff * width + e * f.up_rows * width
     return n
 
 
@@ -674,3 +955,51 @@ def pimodra_layers(n_layers: int, width: int, *, heads: int = 16,
     if loop:
         lp = {"start": loop[0], "stop": loop[1], "times": loop[2]}
     return looped_layer_specs_from_cfg(cfg_layers, lp)
+
+
+def zevilorn_layers(n_layers: int, width: int, *, heads: int = 16,
+                    kv_heads: int = 4, dim: int = 128, window: int = 1024,
+                    kv_rank: int = 512, rot_dim: int = 64, q_rank: int = 768,
+                    gru_width: Optional[int] = None, experts: int = 8,
+                    top_k: int = 2, expert_ff: int = 1024, groups: int = 4,
+                    keep: int = 2, taps: int = 4,
+                    loop: Optional[Tuple[int, int, int]] = None
+                    ) -> List[LayerSpec]:
+    """A synthetic Zevilorn stack for benchmarks: the cycle capped
+    score-mixing attention / latent attention / windowed attention beside a
+    minGRU, every layer with group-routed gelu experts; loop = (start,
+    stop, times) repeats a block with shared tensors."""
+    cfg_layers = []
+    mlp = {"kind": "moe", "expert": {"ff": expert_ff},
+           "router": {"experts": experts, "top": top_k,
+                      "groups": {"count": groups, "keep": keep}}}
+    for i in range(n_layers):
+        k = i % 3
+        if k == 0:
+            typ = "attention"
+            mixer: Dict[str, Any] = {
+                "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim,
+                "scale": dim ** -0.5, "softcap": 50.0, "conv": taps,
+                "mask": {"size": window},
+                "rot": {"base": 1e6, "dims": dim,
+                        "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0,
+                                    "original": 8192}}}
+        elif k == 1:
+            typ = "latent_attention"
+            mixer = {"heads": heads, "dim": dim, "rot_dim": rot_dim,
+                     "vdim": dim, "kv_rank": kv_rank, "q_rank": q_rank,
+                     "scale": (dim + rot_dim) ** -0.5,
+                     "rot": {"base": 1e6, "dims": rot_dim}}
+        else:
+            typ = "parallel"
+            mixer = {"left": {"heads": heads, "kv_heads": kv_heads,
+                              "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                              "mask": {"size": window},
+                              "rot": {"base": 1e6, "dims": dim // 2,
+                                      "scaling": {"factor": 2.0}}},
+                     "right": {"width": gru_width or width}}
+        cfg_layers.append({"type": typ, "mixer": mixer, "mlp": mlp})
+    lp = None
+    if loop:
+        lp = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return gated_layer_specs_from_cfg(cfg_layers, lp)

@@ -48,7 +48,7 @@ class ModelSpec:
     # vocab specials (byte-tokenizer defaults; overridden by a real tokenizer)
     bos_token_id: int = 1
     eos_token_id: int = 2
-    # hybrid stacks (arch "nukopel", "pugozen", "pimodra"): per-layer mixer/feed-forward specs
+    # hybrid stacks (arch "nukopel", "pugozen", "pimodra", "zevilorn"): per-layer mixer/feed-forward specs
     # (models/hybrid.py). When set, the uniform-layer fields above hold
     # representative maxima only; the Runner's hybrid path reads these.
     layer_specs: Optional[List[Any]] = None
@@ -500,6 +500,28 @@ def pimodra_spec(name: str, cfg: Dict[str, Any]) -> ModelSpec:
     return spec
 
 
+def zevilorn_spec(name: str, cfg: Dict[str, Any]) -> ModelSpec:
+    """Parse a Zevilorn config.json dict: gated parallel-form layers with a
+    capped score-mixing attention, a latent attention with a sink, or a
+    windowed attention beside a minGRU; group-routed gelu experts; an
+    optional repeated block of layers (unrolled here into one layer spec per
+    run) before whose later passes the embedding output is added back."""
+    from .hybrid import gated_layer_specs_from_cfg, mixer_parts
+
+    loop = cfg.get("loop") or None
+    layers = gated_layer_specs_from_cfg(cfg["layers"], loop)
+    spec = hybrid_spec(
+        name, int(cfg["vocab"]), int(cfg["width"]), layers,
+        eps=float(cfg["norm"]["eps"]), embed_scale=1.0, canon_taps=0,
+        max_seq_len=int(cfg.get("max_seq_len", 32768)),
+        arch="zevilorn", norm_type="rmsnorm", act_type="gelu",
+    )
+    spec.n_kv_heads = max(getattr(m, "kv_heads", 1) for l in layers
+                          for _, m in mixer_parts(l.mixer))
+    spec.source_cfg = {"layers": cfg["layers"], "loop": loop}
+    return spec
+
+
 def resolve_spec(name: str, model_path: Optional[str] = None) -> ModelSpec:
     """Resolve a model name (preset / alias / HF id / local dir) to a spec.
 
@@ -546,6 +568,9 @@ def spec_from_hf_config(model_path: str, name: Optional[str] = None) -> ModelSpe
             safetensors_shapes(model_path))
     if cfg.get("architecture") == "Pimodra":
         return pimodra_spec(
+            name or os.path.basename(os.path.normpath(model_path)), cfg)
+    if cfg.get("architecture") == "Zevilorn":
+        return zevilorn_spec(
             name or os.path.basename(os.path.normpath(model_path)), cfg)
     if cfg.get("model_type") == "gpt2" or "n_embd" in cfg:
         spec = _gpt2(

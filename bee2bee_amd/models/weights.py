@@ -46,6 +46,8 @@ class LayerWeights:
         # weighted-sandwich layers: the four grouped-norm weights, the
         # attention's head-mixing matrix, the dense activation's numbers
         "norms", "talk", "act_coef",
+        # gated parallel-form layers: the bias of the fused input matrix
+        "b_in",
     )
 
     def __init__(self) -> None:
@@ -79,6 +81,7 @@ class LayerWeights:
         self.norms = None      # 4 x [width] fp32: pre/post mixer, pre/post ffn
         self.talk = None       # [heads, heads] fp32
         self.act_coef = None   # [4] fp32 (PolyNorm a, b, c, e)
+        self.b_in = None       # [in_total] (zeros where a part has no bias)
 
 
 class ModelWeights:
@@ -124,6 +127,8 @@ class ModelWeights:
                 return self._random_init_pugozen(seed)
             if s.arch == "pimodra":
                 return self._random_init_pimodra(seed)
+            if s.arch == "zevilorn":
+                return self._random_init_zevilorn(seed)
             return self._random_init_hybrid(seed)
         lo, hi = layer_range or (0, s.n_layers)
         self.expert_range = expert_range
@@ -225,6 +230,8 @@ class ModelWeights:
                 return self._load_pugozen(model_path)
             if s.arch == "pimodra":
                 return self._load_pimodra(model_path)
+            if s.arch == "zevilorn":
+                return self._load_zevilorn(model_path)
             return self._load_nukopel(model_path)
         if s.arch == "gpt2":
             return self._load_gpt2(model_path, layer_range)
@@ -676,6 +683,207 @@ class ModelWeights:
                 lw.w_gate_up = act(get(p + "mlp.up"))
                 lw.w_down = act(get(p + "mlp.down"))
                 lw.act_coef = f32(get(p + "mlp.act"))
+        for i, l in enumerate(s.layer_specs):
+            if l.weights_of is not None:
+                self.layers[i] = self.layers[l.weights_of]
+
+
+    # --------------------------------------------- gated parallel-form stacks
+
+    @torch.no_grad()
+    def _load_zevilorn(self, model_path: str) -> "ModelWeights":
+        """Zevilorn safetensors: 'embed', 'head', 'final.norm' and per
+        checkpoint layer 'l<i>.norm1', 'l<i>.rg1|rg2' (+ '.b'),
+        'l<i>.mix.*' ('.left.*' / '.right.*' for a parallel mixer),
+        'l<i>.mlp.router|e<k>.up|down'. Linear weights [out, in]; a bias is
+        the weight's name + '.b', a conv the projection's name + '.conv'."""
+        tensors = dict(iter_safetensors(model_path))
+        self._assemble_zevilorn(lambda name: tensors.pop(name))
+        return self
+
+    @torch.no_grad()
+    def _random_init_zevilorn(self, seed: int) -> "ModelWeights":
+        import zlib
+
+        def get(name: str) -> torch.Tensor:
+            tseed = (seed * 1000003 + zlib.crc32(name.encode())) % (2**31)
+            gen = torch.Generator(device=self.device).manual_seed(tseed)
+            shape, mean, std = self._zevilorn_shape(name)
+            t = torch.randn(tuple(shape), generator=gen, dtype=torch.float32,
+                            device=self.device)
+            if name.endswith("mix.talk"):
+                # near the identity: a head keeps most of its own scores
+                t = torch.eye(shape[0], device=self.device) / std + t
+            return (mean + std * t).bfloat16()
+
+        self._assemble_zevilorn(get)
+        return self
+
+    def _zevilorn_shape(self, name: str):
+        """(shape, init mean, init std) of a checkpoint tensor."""
+        s = self.spec
+        W, V = s.hidden_size, s.vocab_size
+        lin = W ** -0.5
+        if name == "embed":
+            return (V, W), 0.0, 1.0
+        if name == "head":
+            return (V, W), 0.0, lin
+        if name == "final.norm":
+            return (W,), 1.0, 0.1
+        head, rest = name.split(".", 1)
+        l = next(x for x in s.layer_specs if x.src == int(head[1:]))
+        f = l.ffn
+        if rest == "norm1":
+            return (W,), 1.0, 0.1
+        if rest in ("rg1", "rg2"):
+            return (W, W), 0.0, lin
+        if rest in ("rg1.b", "rg2.b"):
+            return (W,), 0.0, 0.5
+        if rest == "mlp.router":
+            return (f.n_experts, W), 0.0, lin
+        if rest.startswith("mlp."):
+            if rest.endswith(".down"):
+                return (W, f.ff), 0.0, f.ff ** -0.5
+            return (f.up_rows, W), 0.0, lin
+        rest = rest[len("mix."):]
+        m = l.mixer
+        if m.kind == "parallel":
+            if rest in ("left.out", "right.out"):
+                return (W,), 1.0, 0.1
+            side, rest = rest.split(".", 1)
+            m = m.left if side == "left" else m.right
+        if rest == "o":
+            return (W, m.out_size), 0.0, m.out_size ** -0.5
+        if rest == "o.b":
+            return (W,), 0.0, 0.1
+        sizes = dict(m.in_sizes)
+        if m.kind == "latent_attention":
+            table = {"dq": ((m.q_rank, W), 0.0, lin),
+                     "q": ((m.q_size, W), 0.0, lin),
+                     "dq.norm": ((m.q_rank,), 1.0, 0.1),
+                     "uq": ((m.q_size, max(1, m.q_rank)), 0.0,
+                            max(1, m.q_rank) ** -0.5),
+                     "dkv": ((m.cache_dim, W), 0.0, lin),
+                     "dkv.norm": ((m.kv_rank,), 1.0, 0.1),
+                     "uk": ((m.heads * m.dim, m.kv_rank), 0.0,
+                            m.kv_rank ** -0.5),
+                     "uv": ((m.heads * m.vdim, m.kv_rank), 0.0,
+                            m.kv_rank ** -0.5),
+                     "sink": ((m.heads,), 0.0, 1.0),
+                     "g": ((m.heads, W), 0.0, lin)}
+            return table[rest]
+        if m.kind == "gqa_attention" and rest == "talk":
+            return (m.heads, m.heads), 0.0, 0.1
+        if rest.endswith(".conv"):
+            return (sizes[rest[:-5]], m.taps), 0.0, 0.4
+        if rest.endswith(".b"):
+            return (sizes[rest[:-2]],), 0.0, 0.1
+        return (sizes[rest], W), 0.0, lin
+
+    def _assemble_zevilorn(self, get) -> None:
+        """Engine layout of a gated parallel-form stack: per layer ONE
+        input matrix with every projection that reads the normed h (the
+        mixer's and the two residual gates; models/hybrid.py gated_layout)
+        and its bias vector, output projections per mixer part, the latent
+        attention's per-head up-projection stacks, stacked expert matrices
+        [E, ff, W] / [E, W, ff]; norm weights, conv taps (tap-major), the
+        score-mixing matrix, sinks and the router in fp32. A run with
+        weights_of shares the owning run's LayerWeights."""
+        from types import SimpleNamespace
+
+        from .hybrid import gated_layout, mixer_parts
+
+        s = self.spec
+        dev, dt = self.device, self.dtype
+        W = s.hidden_size
+
+        def act(t: torch.Tensor) -> torch.Tensor:
+            return t.to(dev, dt).contiguous()
+
+        def f32(t: torch.Tensor) -> torch.Tensor:
+            return t.to(dev, torch.float32).contiguous()
+
+        self.embed = act(get("embed"))
+        self.lm_head = act(get("head"))
+        self.final_norm = f32(get("final.norm"))
+        for i, l in enumerate(s.layer_specs):
+            if l.weights_of is not None:
+                continue
+            lw, p = self.layers[i], f"l{l.src}."
+            ins, n_in = gated_layout(l, W)
+            lw.layout = (ins, n_in)
+            lw.norm_w = f32(get(p + "norm1"))
+            w_in = torch.zeros(n_in, W, device=dev, dtype=dt)
+            b_in = torch.zeros(n_in, device=dev, dtype=dt)
+
+            def put_in(key: str, name: str, bias: bool = False) -> None:
+                off, n = ins[key]
+                t = get(name)
+                assert t.shape == (n, W), (name, tuple(t.shape), n)
+                w_in[off : off + n] = t.to(dev, dt)
+                if bias:
+                    b_in[off : off + n] = get(name + ".b").to(dev, dt)
+
+            lw.mix = {}
+            for pre, m in mixer_parts(l.mixer):
+                q = p + "mix." + pre
+                ns = lw.mix[pre] = SimpleNamespace()
+                if m.kind == "gqa_attention":
+                    for n_ in ("q", "k", "v"):
+                        put_in(pre + n_, q + n_, m.bias)
+                    if m.head_gate:
+                        put_in(pre + "g", q + "g")
+                    # checkpoint [channels, taps] -> tap-major [taps, channels]
+                    ns.conv_w = f32(torch.cat(
+                        [get(q + "q.conv"), get(q + "k.conv"),
+                         get(q + "v.conv")], dim=0).t()) if m.taps > 1 else None
+                    if m.taps == 1:
+                        # a single tap carries nothing: fold it into the rows
+                        for n_ in ("q", "k", "v"):
+                            off, n = ins[pre + n_]
+                            tap = get(q + n_ + ".conv").to(dev, torch.float32)
+                            w_in[off : off + n] = (
+                                w_in[off : off + n].float() * tap).to(dt)
+                            b_in[off : off + n] = (
+                                b_in[off : off + n].float() * tap[:, 0]).to(dt)
+                    ns.talk = f32(get(q + "talk")) if m.score_mix else None
+                    ns.wo_b = act(get(q + "o.b")) if m.bias else None
+                elif m.kind == "latent_attention":
+                    if m.q_rank:
+                        put_in(pre + "dq", q + "dq")
+                        ns.q_norm = f32(get(q + "dq.norm"))
+                        ns.w_uq = act(get(q + "uq"))
+                    else:
+                        put_in(pre + "q", q + "q")
+                        ns.q_norm = ns.w_uq = None
+                    put_in(pre + "dkv", q + "dkv")
+                    put_in(pre + "g", q + "g")
+                    ns.kv_norm = f32(get(q + "dkv.norm"))
+                    ns.w_uk = act(get(q + "uk").reshape(
+                        m.heads, m.dim, m.kv_rank))
+                    ns.w_uv = act(get(q + "uv").reshape(
+                        m.heads, m.vdim, m.kv_rank).transpose(1, 2))
+                    ns.sink = f32(get(q + "sink")) if m.sink else None
+                    ns.wo_b = None
+                else:
+                    put_in(pre + "z", q + "z", True)
+                    put_in(pre + "x", q + "x", True)
+                    put_in(pre + "g", q + "g")
+                    ns.wo_b = None
+                ns.wo = act(get(q + "o"))
+                if l.mixer.kind == "parallel" and \
+                        l.mixer.combine == "normed_mean":
+                    ns.out_norm = f32(get(p + "mix." + pre + "out"))
+            put_in("rg1", p + "rg1", True)
+            f = l.ffn
+            if f is not None:
+                put_in("rg2", p + "rg2", True)
+                lw.moe_gate = f32(get(p + "mlp.router"))
+                lw.moe_w_gate_up = act(torch.stack([
+                    get(f"{p}mlp.e{e}.up") for e in range(f.n_experts)]))
+                lw.moe_w_down = act(torch.stack([
+                    get(f"{p}mlp.e{e}.down") for e in range(f.n_experts)]))
+            lw.w_in, lw.b_in = w_in, b_in
         for i, l in enumerate(s.layer_specs):
             if l.weights_of is not None:
                 self.layers[i] = self.layers[l.weights_of]

@@ -285,15 +285,20 @@ def latent_rope_store(q_rot, kv, kv_norm, eps: float, kv_rank: int,
 
 
 def latent_attn(q_abs, q_rot, gate, cache, block_table, positions, seq_idx,
-                cu_seqlens, window: int, scale: float, max_qlen: int = 0):
+                cu_seqlens, window: int, scale: float, max_qlen: int = 0,
+                sink=None):
     """max_qlen: longest chunk in the batch (host int); 1 selects the
-    decode kernel, larger the query-tiled prefill kernel."""
+    decode kernel, larger the query-tiled prefill kernel. window 0: every
+    earlier position; sink fp32 [heads]: a logit per head in the softmax
+    denominator."""
     if _use_hip(q_abs):
         return require_hip().latent_attn(q_abs, q_rot, gate, cache,
                                          block_table, positions, seq_idx,
-                                         cu_seqlens, window, scale, max_qlen)
+                                         cu_seqlens, window, scale, max_qlen,
+                                         sink)
     return reference.latent_attn(q_abs, q_rot, gate, cache, block_table,
-                                 positions, seq_idx, cu_seqlens, window, scale)
+                                 positions, seq_idx, cu_seqlens, window, scale,
+                                 sink)
 
 
 def lightning_attn(q, k, v, decay, state, state_slots, cu_seqlens, positions,
@@ -477,6 +482,79 @@ def silu_glu(gate_up):
     return reference.silu_glu(gate_up)
 
 
-def group_topk_gate(logits, top_k: int, n_groups: int, keep_groups: int):
+def group_topk_gate(logits, top_k: int, n_groups: int, keep_groups: int,
+                    score: str = "softmax", group_top: int = 1):
     # [T, E] gating math: torch ops on both devices, like moe_topk_gate
-    return reference.group_topk_gate(logits, top_k, n_groups, keep_groups)
+    return reference.group_topk_gate(logits, top_k, n_groups, keep_groups,
+                                     score, group_top)
+
+
+# ------------------------------------------- gated parallel-form stacks
+# (ops/reference.py documents shapes and formulas)
+
+rope_freq_tables = reference.rope_freq_tables
+
+
+def rope_store(q, k, v, q_out, rope_dims: int, interleaved: bool, positions,
+               cos, sin, q_mult: float, k_cache, v_cache,
+               slot_mapping) -> None:
+    if _use_hip(q_out):
+        require_hip().rope_store(q, k, v, q_out, rope_dims, interleaved,
+                                 positions, cos, sin, float(q_mult), k_cache,
+                                 v_cache, slot_mapping)
+        return
+    reference.rope_store(q, k, v, q_out, rope_dims, interleaved, positions,
+                         cos, sin, q_mult, k_cache, v_cache, slot_mapping)
+
+
+def gqa_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
+             cu_seqlens, softcap: float, talk, sink, head_gate, window: int,
+             out, max_qlen: int = 0) -> None:
+    """max_qlen: longest chunk of the step (host int). Without a cap and a
+    score mix the step runs on the sink-attention kernels (matrix cores for
+    bf16 prompt portions); with them, on the score-mixing kernels."""
+    if _use_hip(q):
+        require_hip().gqa_attn(q, k_cache, v_cache, block_table, positions,
+                               seq_idx, cu_seqlens, float(softcap), talk,
+                               sink, head_gate, window, out, max_qlen)
+        return
+    reference.gqa_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
+                       cu_seqlens, softcap, talk, sink, head_gate, window, out)
+
+
+def min_gru(z, x, g, state, state_slots, cu_seqlens, positions, out,
+            max_qlen: int = 0) -> None:
+    if _use_hip(z):
+        require_hip().min_gru(z, x, g, state, state_slots, cu_seqlens,
+                              positions, out, max_qlen)
+        return
+    reference.min_gru(z, x, g, state, state_slots, cu_seqlens, positions, out)
+
+
+def pair_rmsnorm_mean(a, wa, b, wb, eps: float, out_dtype):
+    if _use_hip(a):
+        return require_hip().pair_rmsnorm_mean(a, wa, b, wb, eps, out_dtype)
+    return reference.pair_rmsnorm_mean(a, wa, b, wb, eps, out_dtype)
+
+
+def slice_rmsnorm(x, w, eps: float):
+    if _use_hip(x):
+        return require_hip().slice_rmsnorm(x, w, eps)
+    return reference.slice_rmsnorm(x, w, eps)
+
+
+def gated_add_rmsnorm(resid, y1, g1, y2, g2, extra, w, eps: float,
+                      out_dtype):
+    """resid(fp32) += sigmoid(g1) y1 [+ sigmoid(g2) y2] [+ extra] in place;
+    -> unit(resid) * w (None when w is None). One pass on the GPU."""
+    if _use_hip(resid):
+        return require_hip().gated_add_rmsnorm(resid, y1, g1, y2, g2, extra,
+                                               w, eps, out_dtype)
+    return reference.gated_add_rmsnorm(resid, y1, g1, y2, g2, extra, w, eps,
+                                       out_dtype)
+
+
+def gelu_erf(x):
+    if _use_hip(x):
+        return require_hip().gelu_erf(x)
+    return reference.gelu_erf(x)

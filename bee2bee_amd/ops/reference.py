@@ -422,12 +422,15 @@ def latent_attn(q_abs: torch.Tensor, q_rot: torch.Tensor, gate: torch.Tensor,
                 cache: torch.Tensor, block_table: torch.Tensor,
                 positions: torch.Tensor, seq_idx: torch.Tensor,
                 cu_seqlens: torch.Tensor, window: int,
-                scale: float) -> torch.Tensor:
+                scale: float,
+                sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Windowed softmax attention in the latent space (one shared key/value
     row per token). q_abs [H, T, C] (queries already multiplied by the key
     up-projection), q_rot [T, H, R], gate [T, H] raw (sigmoid applied here).
     Row t at position p of sequence b sees cached positions
-    max(0, p - window + 1) .. p. Returns [H, T, C] in q_abs.dtype."""
+    max(0, p - window + 1) .. p (window 0: 0 .. p). sink fp32 [H]: exp(sink)
+    joins the softmax denominator, unscaled, without a value. Returns
+    [H, T, C] in q_abs.dtype."""
     H, T, C = q_abs.shape
     bs = cache.shape[1]
     flat = cache.view(-1, cache.shape[-1])
@@ -438,7 +441,7 @@ def latent_attn(q_abs: torch.Tensor, q_rot: torch.Tensor, gate: torch.Tensor,
         if hi == lo:
             continue
         pos = positions[lo:hi].long()
-        k_lo = max(0, int(pos.min()) - window + 1)
+        k_lo = max(0, int(pos.min()) - window + 1) if window > 0 else 0
         k_hi = int(pos.max()) + 1
         kpos = torch.arange(k_lo, k_hi, device=q_abs.device)
         rows = block_table[b].long()[kpos // bs] * bs + kpos % bs
@@ -447,8 +450,17 @@ def latent_attn(q_abs: torch.Tensor, q_rot: torch.Tensor, gate: torch.Tensor,
         s += torch.einsum("thr,sr->hts", q_rot[lo:hi].float(), kv[:, C:])
         s *= scale
         d = pos[:, None] - kpos[None, :]
-        s.masked_fill_(((d < 0) | (d >= window))[None], float("-inf"))
-        p = torch.softmax(s, dim=-1)
+        dead = d < 0
+        if window > 0:
+            dead = dead | (d >= window)
+        s.masked_fill_(dead[None], float("-inf"))
+        if sink is None:
+            p = torch.softmax(s, dim=-1)
+        else:
+            sk = sink.float().view(H, 1, 1)
+            m = torch.maximum(s.max(-1, keepdim=True).values, sk)
+            e = torch.exp(s - m)
+            p = e / (e.sum(-1, keepdim=True) + torch.exp(sk - m))
         o = torch.einsum("hts,sc->htc", p, kv[:, :C])
         out[:, lo:hi] = o * torch.sigmoid(gate[lo:hi].float()).t()[..., None]
     return out.to(q_abs.dtype)
@@ -981,18 +993,28 @@ def silu_glu(gate_up: torch.Tensor) -> torch.Tensor:
 
 
 def group_topk_gate(logits: torch.Tensor, top_k: int, n_groups: int,
-                    keep_groups: int) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Group-limited choice on softmax scores. logits fp32 [T, E]: scores =
-    softmax over all experts; experts form n_groups equal groups of
-    neighbours, a group's score is its largest expert score, experts outside
+                    keep_groups: int, score: str = "softmax",
+                    group_top: int = 1) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Group-limited choice on expert scores. logits fp32 [T, E]: scores =
+    softmax over all experts (score "softmax") or the sigmoid of each logit
+    ("sigmoid"); experts form n_groups equal groups of neighbours, a group's
+    score is the sum of its group_top largest expert scores, experts outside
     the best keep_groups groups cannot be chosen; the top_k remaining scores
     are the weights, as they are. -> (weights [T, k] fp32, idx [T, k] int32).
     Fixed shapes and no host sync (graph-capturable)."""
     T, E = logits.shape
-    s = torch.softmax(logits.float(), dim=-1)
+    if score == "sigmoid":
+        s = torch.sigmoid(logits.float())
+    else:
+        s = torch.softmax(logits.float(), dim=-1)
     pick = s
     if n_groups > 1 and keep_groups < n_groups:
-        gs = s.view(T, n_groups, E // n_groups).max(-1).values
+        per = s.view(T, n_groups, E // n_groups)
+        if group_top <= 1:
+            gs = per.max(-1).values
+        else:
+            gs = torch.topk(per, min(group_top, E // n_groups),
+                            dim=-1).values.sum(-1)
         top_g = torch.topk(gs, keep_groups, dim=-1).indices
         allow = torch.zeros(T, n_groups, dtype=torch.bool, device=s.device)
         allow.scatter_(1, top_g, True)
@@ -1000,3 +1022,214 @@ def group_topk_gate(logits: torch.Tensor, top_k: int, n_groups: int,
         pick = torch.where(allow.reshape(T, E), s, torch.full_like(s, -1.0))
     idx = torch.topk(pick, top_k, dim=-1).indices
     return s.gather(1, idx), idx.to(torch.int32)
+
+
+# ------------------------------------------- gated parallel-form stacks
+#
+# Mechanisms of stacks whose layers are
+#   x += sigmoid(g1) * mixer(h) + sigmoid(g2) * ffn(h),  h = unit(x) * w:
+# the gated residual update fused with the next norm, rotation tables with a
+# linear or banded frequency scaling, rotation in either pair layout with the
+# page store, grouped-query attention with capped, head-mixed scores, the
+# minGRU recurrence, the mean of two normed branch outputs, a norm on a
+# column slice, the exact gelu.
+
+
+def rope_freq_tables(max_len: int, dims: int, base: float,
+                     scaling: Optional[dict], device
+                     ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """cos/sin [max_len, dims/2], float64 angles rounded once to fp32. Pair
+    i turns at f_i = base^(-2i/dims). scaling {"kind": "linear", factor}:
+    f_i / factor. {"kind": "banded", factor, low, high, original}: with
+    wavelength l = 2 pi / f_i, f_i is kept where l < original / high,
+    divided by factor where l > original / low, and in between blended,
+    (1 - s) f_i / factor + s f_i with s = (original / l - low) /
+    (high - low)."""
+    half = dims // 2
+    i = torch.arange(half, dtype=torch.float64)
+    inv = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                    -2.0 * i / dims)
+    if scaling:
+        factor = float(scaling["factor"])
+        if scaling.get("kind", "linear") == "linear":
+            inv = inv / factor
+        else:
+            lo, hi = float(scaling["low"]), float(scaling["high"])
+            orig = float(scaling["original"])
+            wl = 2.0 * math.pi / inv
+            sm = ((orig / wl - lo) / (hi - lo)) if hi != lo else \
+                torch.ones_like(wl)
+            blend = (1.0 - sm) * inv / factor + sm * inv
+            inv = torch.where(wl < orig / hi, inv,
+                              torch.where(wl > orig / lo, inv / factor, blend))
+    ang = torch.outer(torch.arange(max_len, dtype=torch.float64), inv)
+    return (ang.cos().to(device, torch.float32),
+            ang.sin().to(device, torch.float32))
+
+
+def _rot_pairs(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+               dims: int) -> torch.Tensor:
+    """Rotate the first `dims` coords of x [..., D], pairing 2i with 2i+1;
+    cos/sin broadcast against x[..., :dims:2]."""
+    u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+    rot = torch.stack([u * cos - v * sin, v * cos + u * sin], -1)
+    return torch.cat([rot.flatten(-2), x[..., dims:]], -1)
+
+
+def rope_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+               q_out: torch.Tensor, rope_dims: int, interleaved: bool,
+               positions: torch.Tensor, cos, sin, q_mult: float,
+               k_cache: torch.Tensor, v_cache: torch.Tensor,
+               slot_mapping: torch.Tensor) -> None:
+    """q [T, H, D], k [T, G, D], v [T, G, Dv] (views, any float dtype, left
+    as they are unless q_out aliases q): rotate(q) * q_mult -> q_out
+    [T, H, D]; rotate(k) -> k_cache [n_blocks, G, block, D]; v -> v_cache
+    [n_blocks, G, block, Dv], at slot_mapping. The rotation covers the first
+    rope_dims coordinates, pairs (2i, 2i+1) when interleaved, else
+    (i, i + rope_dims/2)."""
+    bs = k_cache.shape[2]
+    qf, kf = q.float(), k.float()
+    if rope_dims:
+        p = positions.long()
+        c, s = cos[p][:, None], sin[p][:, None]
+        rot = _rot_pairs if interleaved else _rot_half
+        qf, kf = rot(qf, c, s, rope_dims), rot(kf, c, s, rope_dims)
+    q_out.copy_((qf * q_mult).to(q_out.dtype))
+    slot = slot_mapping.long()
+    blk, off = slot // bs, slot % bs
+    k_cache[blk, :, off] = kf.to(k_cache.dtype)
+    v_cache[blk, :, off] = v.to(v_cache.dtype)
+
+
+def gqa_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+             block_table: torch.Tensor, positions: torch.Tensor,
+             seq_idx: torch.Tensor, cu_seqlens: torch.Tensor,
+             softcap: float, talk: Optional[torch.Tensor],
+             sink: Optional[torch.Tensor],
+             head_gate: Optional[torch.Tensor], window: int,
+             out: torch.Tensor) -> None:
+    """Grouped-query attention over the pages. Scores q . k (the score
+    scale is already in q); softcap > 0: s <- softcap tanh(s / softcap);
+    talk fp32 [H, H]: s_h <- sum_g talk[h, g] s_g at every (row, key),
+    BEFORE the softmax. Row t at position p of chunk b sees cached positions
+    j <= p (j > p - window when window > 0). sink fp32 [H]: exp(sink_h)
+    joins the denominator without a value. head_gate [T, H] raw (strided
+    view): head h's output times sigmoid(head_gate[t, h]).
+    out [T, H * Dv] (strided view)."""
+    T, H, D = q.shape
+    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    rep = H // G
+    cu = cu_seqlens.tolist()
+    res = torch.zeros(T, H, Dv, dtype=torch.float32, device=q.device)
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        pos = positions[lo:hi].long()
+        k_lo = max(0, int(pos.min()) - window + 1) if window > 0 else 0
+        k_hi = int(pos.max()) + 1
+        kpos = torch.arange(k_lo, k_hi, device=q.device)
+        blk = block_table[b].long()[kpos // bs]
+        keys = k_cache[blk, :, kpos % bs].float()          # [S, G, D]
+        vals = v_cache[blk, :, kpos % bs].float()          # [S, G, Dv]
+        qb = q[lo:hi].float().view(hi - lo, G, rep, D)
+        s = torch.einsum("tgrd,sgd->grts", qb, keys).reshape(H, hi - lo, -1)
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        if talk is not None:
+            s = torch.einsum("hg,gts->hts", talk.float(), s)
+        d = pos[:, None] - kpos[None, :]
+        dead = d < 0
+        if window > 0:
+            dead = dead | (d >= window)
+        s = s.masked_fill(dead[None], float("-inf"))
+        m = s.max(-1, keepdim=True).values
+        if sink is not None:
+            sk = sink.float().view(H, 1, 1)
+            m = torch.maximum(m, sk)
+        e = torch.exp(s - m)
+        den = e.sum(-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(sk - m)
+        w = (e / den).view(G, rep, hi - lo, -1)
+        o = torch.einsum("grts,sgv->tgrv", w, vals)
+        res[lo:hi] = o.reshape(hi - lo, H, Dv)
+    if head_gate is not None:
+        res = res * torch.sigmoid(head_gate.float())[..., None]
+    out.copy_(res.view(T, H * Dv).to(out.dtype))
+
+
+def min_gru(z: torch.Tensor, x: torch.Tensor, g: torch.Tensor,
+            state: torch.Tensor, state_slots: torch.Tensor,
+            cu_seqlens: torch.Tensor, positions: torch.Tensor,
+            out: torch.Tensor) -> None:
+    """Element-wise gated recurrence over packed chunks, fp32 inside.
+    z, x, g [T, N] raw projections (strided views): a = sigmoid(z),
+    c = x + 1/2 where x >= 0 else sigmoid(x), S_t = (1 - a) S_(t-1) + a c,
+    out [T, N] (strided view) <- S_t * silu(g). state [n_slots, N] fp32 is
+    read unless the chunk starts at position 0 and advanced in place."""
+    a = torch.sigmoid(z.float())
+    xf = x.float()
+    c = torch.where(xf >= 0, xf + 0.5, torch.sigmoid(xf))
+    gate = torch.nn.functional.silu(g.float())
+    res = torch.empty_like(xf)
+    cu = cu_seqlens.tolist()
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        slot = int(state_slots[b])
+        if int(positions[lo]) == 0:
+            S = torch.zeros_like(xf[0])
+        else:
+            S = state[slot].clone()
+        for t in range(lo, hi):
+            S = (1.0 - a[t]) * S + a[t] * c[t]
+            res[t] = S
+        state[slot] = S
+    out.copy_((res * gate).to(out.dtype))
+
+
+def pair_rmsnorm_mean(a: torch.Tensor, wa: torch.Tensor, b: torch.Tensor,
+                      wb: torch.Tensor, eps: float,
+                      out_dtype: torch.dtype) -> torch.Tensor:
+    """(unit(a) * wa + unit(b) * wb) / 2 over rows [T, W]."""
+    def un(x):
+        xf = x.float()
+        return xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+
+    return (0.5 * (un(a) * wa.float() + un(b) * wb.float())).to(out_dtype)
+
+
+def slice_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float
+                  ) -> torch.Tensor:
+    """unit(x) * w for rows [T, N] that may be a strided column slice;
+    contiguous result in x.dtype."""
+    xf = x.float()
+    r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (xf * r * w.float()).to(x.dtype).contiguous()
+
+
+def gated_add_rmsnorm(resid: torch.Tensor, y1: torch.Tensor,
+                      g1: torch.Tensor, y2: Optional[torch.Tensor],
+                      g2: Optional[torch.Tensor],
+                      extra: Optional[torch.Tensor],
+                      w: Optional[torch.Tensor], eps: float,
+                      out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """resid (fp32, in place) += sigmoid(g1) * y1 [+ sigmoid(g2) * y2]
+    [+ extra]; returns unit(resid) * w (None if w is). g1, g2 [T, W] raw
+    (strided views); extra [T, W]. y1 None: only extra and the norm."""
+    if y1 is not None:
+        resid.add_(torch.sigmoid(g1.float()) * y1.float())
+    if y2 is not None:
+        resid.add_(torch.sigmoid(g2.float()) * y2.float())
+    if extra is not None:
+        resid.add_(extra.float())
+    if w is None:
+        return None
+    return rmsnorm_f32(resid, w, eps, out_dtype)
+
+
+def gelu_erf(x: torch.Tensor) -> torch.Tensor:
+    """Exact gelu, x/2 (1 + erf(x / sqrt 2)), evaluated in fp32."""
+    return torch.nn.functional.gelu(x.float()).to(x.dtype)
