@@ -514,9 +514,17 @@ def gqa_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
     score mix the step runs on the sink-attention kernels (matrix cores for
     bf16 prompt portions); with them, on the score-mixing kernels."""
     if _use_hip(q):
-        require_hip().gqa_attn(q, k_cache, v_cache, block_table, positions,
-                               seq_idx, cu_seqlens, float(softcap), talk,
-                               sink, head_gate, window, out, max_qlen)
+        if talk is None and not softcap:
+            require_hip().sink_attn(q, k_cache, v_cache, block_table,
+                                    positions, seq_idx, cu_seqlens, sink,
+                                    window, out, 1.0, max_qlen, head_gate)
+        else:
+            if talk is None:    # a cap alone: mix with the identity
+                talk = torch.eye(q.shape[1], dtype=torch.float32,
+                                 device=q.device)
+            require_hip().mixed_score_attn(q, k_cache, v_cache, block_table,
+                                           positions, seq_idx, float(softcap),
+                                           talk, sink, head_gate, window, out)
         return
     reference.gqa_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
                        cu_seqlens, softcap, talk, sink, head_gate, window, out)

@@ -138,7 +138,10 @@ __global__ __launch_bounds__(64) void attn_prefill_basic(
 // whose attention weights are 32-bit quantities. sink (optional, [nq] fp32):
 // a per-head logit counted once in the softmax denominator, with no key and
 // no value. The output row of token t, head h starts at out + t*s_o + h*HD
-// and is multiplied by out_scale.
+// and is multiplied by out_scale. window > 0: the row at absolute position
+// p sees keys p - window < j <= p, and key tiles wholly before the tile's
+// first window are skipped. head_gate (optional, bf16 [tokens, nq] with row
+// stride s_g): head h's output times sigmoid(head_gate[t, h]).
 template <int HD, bool PAGED, typename KVT, bool HILO = false>
 __global__ __launch_bounds__(256) void attn_prefill_mfma(
     const unsigned short* __restrict__ q,
@@ -149,7 +152,9 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
     const int* __restrict__ seq_lens,      // PAGED only
     unsigned short* __restrict__ out,
     int nq, int nkv, long s_q, long s_k, long s_v, int W, int bs,
-    float scale, const float* __restrict__ sink, float out_scale, long s_o) {
+    float scale, const float* __restrict__ sink, float out_scale, long s_o,
+    int window = 0, const unsigned short* __restrict__ head_gate = nullptr,
+    long s_g = 0) {
     constexpr int KSTEPS = HD / 32;
     const int seq = blockIdx.z;
     const int h = blockIdx.y;
@@ -214,8 +219,11 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
 
     // causal: keys up to the last absolute q position of this tile
     const int kv_end = min(L, hist + q0 + PF_TM);
+    // window: the tile's first row is the one that reaches back farthest
+    const int kv_lo =
+        window > 0 ? max(0, hist + q0 - window + 1) / PF_TN * PF_TN : 0;
 
-    for (int kb = 0; kb < kv_end; kb += PF_TN) {
+    for (int kb = kv_lo; kb < kv_end; kb += PF_TN) {
         // ---- stage K tile [32][HD] and V^T tile [HD][32]
         __syncthreads();
         {
@@ -274,7 +282,8 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
             for (int r = 0; r < 4; ++r) {
                 const int qrow = q0 + wid * PF_QROWS + lg * 4 + r;
                 const int key = kb + f * 16 + li;
-                if (key > hist + qrow || qrow >= QL || key >= kv_end)
+                if (key > hist + qrow || qrow >= QL || key >= kv_end ||
+                    (window > 0 && key <= hist + qrow - window))
                     sfrag[f][r] = -1e30f;
                 pmax[r] = fmaxf(pmax[r], sfrag[f][r]);
             }
@@ -369,6 +378,8 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
             lsum = lsum * e + __expf(sk - M);
             w *= e;
         }
+        if (head_gate)
+            w /= 1.f + __expf(-bf2f(head_gate[(long)(s0 + qrow) * s_g + h]));
         const float inv = (lsum > 0.f) ? w / lsum : 0.f;
         unsigned short* orow = out + (long)(s0 + qrow) * s_o + (long)h * HD;
 #pragma unroll
@@ -459,13 +470,15 @@ extern "C" void launch_attn_prefill_paged(
 // weights (bf16 hi+lo pair), an optional per-head sink logit, an output
 // scale and a strided output (a column slice of a wider buffer). bf16,
 // head size 64 or 128 (returns nonzero otherwise); scale is applied by the
-// caller (folded into q).
+// caller (folded into q). window 0: causal without a window; head_gate
+// optional (see the kernel).
 extern "C" int launch_attn_prefill_paged_sink(
     const unsigned short* q, long s_q, const unsigned short* k_cache,
     const unsigned short* v_cache, const int* cu, const int* block_table,
     const int* seq_lens, unsigned short* out, long s_o, int nseq, int nq,
     int nkv, int hd, int W, int bs, int max_qlen, const float* sink,
-    float out_scale, hipStream_t stream) {
+    float out_scale, int window, const unsigned short* head_gate, long s_g,
+    hipStream_t stream) {
     if (hd != 64 && hd != 128) return 1;
     if (nseq == 0 || max_qlen == 0) return 0;
     const int tiles = (max_qlen + PF_TM - 1) / PF_TM;
@@ -476,13 +489,13 @@ extern "C" int launch_attn_prefill_paged_sink(
             (attn_prefill_mfma<128, true, unsigned short, true>), grid,
             dim3(256), smem, stream, q, k_cache, v_cache, cu, block_table,
             seq_lens, out, nq, nkv, s_q, 0, 0, W, bs, 1.f, sink, out_scale,
-            s_o);
+            s_o, window, head_gate, s_g);
     else
         hipLaunchKernelGGL(
             (attn_prefill_mfma<64, true, unsigned short, true>), grid,
             dim3(256), smem, stream, q, k_cache, v_cache, cu, block_table,
             seq_lens, out, nq, nkv, s_q, 0, 0, W, bs, 1.f, sink, out_scale,
-            s_o);
+            s_o, window, head_gate, s_g);
     return 0;
 }
 

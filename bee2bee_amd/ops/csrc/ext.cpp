@@ -397,10 +397,12 @@ void bw_probe(const Tensor& pool, int64_t mode, int64_t hd, int64_t arg) {
 
 void register_hybrid_ops(pybind11::module_& m);  // hybrid_ext.cpp
 void register_sandwich_ops(pybind11::module_& m);  // sandwich_ext.cpp
+void register_gated_ops(pybind11::module_& m);  // gated_ext.cpp
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     register_hybrid_ops(m);
     register_sandwich_ops(m);
+    register_gated_ops(m);
     m.def("rmsnorm", &rmsnorm, "fused RMSNorm (bf16)");
     m.def("fused_add_rmsnorm", &fused_add_rmsnorm,
           "residual += x; y = rmsnorm(residual)");

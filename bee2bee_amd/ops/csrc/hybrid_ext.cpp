@@ -33,12 +33,12 @@ void launch_latent_rope_store(void*, long, long, int, const void*, long,
 int launch_latent_attn(const void*, const void*, long, long, const void*,
                        long, const void*, const int*, int, const int*,
                        const int*, void*, float*, float*, int, int, int, int,
-                       int, int, int, float, int, hipStream_t);
+                       int, int, int, float, int, const float*, hipStream_t);
 int launch_latent_attn_mfma(const void*, const void*, long, long, const void*,
                             long, const void*, const int*, int, const int*,
                             const int*, const int*, void*, float*, float*,
                             int, int, int, int, int, int, int, int, int,
-                            float, hipStream_t);
+                            float, const float*, hipStream_t);
 int lightning_segment_tokens();
 int launch_lightning(const void*, const void*, const void*, long,
                      const float*, float*, const int*, const int*, const int*,
@@ -71,11 +71,12 @@ int launch_attn_prefill_paged_sink(const unsigned short*, long,
                                    const unsigned short*, const int*,
                                    const int*, const int*, unsigned short*,
                                    long, int, int, int, int, int, int, int,
-                                   const float*, float, hipStream_t);
+                                   const float*, float, int,
+                                   const unsigned short*, long, hipStream_t);
 int launch_sink_attn(const void*, long, const void*, const void*, const int*,
                      int, const int*, const int*, const float*, void*, long,
                      float, float*, float*, int, int, int, int, int, int, int,
-                     int, int, hipStream_t);
+                     int, int, const void*, long, hipStream_t);
 }
 
 namespace {
@@ -250,7 +251,8 @@ Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
                    const Tensor& gate, const Tensor& cache,
                    const Tensor& block_table, const Tensor& positions,
                    const Tensor& seq_idx, const Tensor& cu, int64_t window,
-                   double scale, int64_t max_qlen) {
+                   double scale, int64_t max_qlen,
+                   const std::optional<Tensor>& sink) {
     const int c = act_code(q_abs, "q_abs");
     check_i32(cu, "cu_seqlens");
     check_i32(block_table, "block_table");
@@ -270,8 +272,19 @@ Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
                 cache.is_contiguous() && cache.dim() == 3 &&
                 cache.size(2) == C + R);
     TORCH_CHECK(block_table.dim() == 2 && positions.numel() == Tn &&
-                seq_idx.numel() == Tn && window >= 1);
+                seq_idx.numel() == Tn && window >= 0);
+    // window 0: every earlier position (a window no context reaches)
+    if (window == 0) window = 1 << 30;
+    const float* sk = nullptr;
+    if (sink.has_value()) {
+        check_f32(*sink, "sink");
+        TORCH_CHECK(sink->numel() == H);
+        sk = sink->data_ptr<float>();
+    }
     Tensor out = torch::empty_like(q_abs);
+    // the most keys a row can see
+    const long reach =
+        std::min<long>(window, block_table.size(1) * cache.size(1));
     auto f32opt = q_abs.options().dtype(torch::kFloat32);
     Tensor part_acc, part_ml;
     float *pa = nullptr, *pm = nullptr;
@@ -290,7 +303,7 @@ Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
         if (max_qlen == 1) {
             // one resident round: 3 workgroups fit a CU's LDS, 256 CUs
             sp = 768 / std::max<long>(1, (long)Tn * ((H + 15) / 16));
-            sp = std::max<long>(1, std::min<long>({sp, 16, (window + 63) / 64}));
+            sp = std::max<long>(1, std::min<long>({sp, 16, (reach + 63) / 64}));
             if (sp > 1) alloc_parts(sp);
         }
         const int rc = launch_latent_attn_mfma(
@@ -301,7 +314,7 @@ Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
             positions.data_ptr<int>(), seq_idx.data_ptr<int>(),
             out.data_ptr(), pa, pm, (int)sp, Tn, (int)cu.numel() - 1,
             (int)max_qlen, H, C, R, (int)cache.size(1), (int)window,
-            (float)scale, stream());
+            (float)scale, sk, stream());
         TORCH_CHECK(rc == 0, "latent_attn: matrix-core path refused a shape "
                              "its guard admitted");
         return out;
@@ -309,7 +322,7 @@ Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
     // few rows: split each row's keys over more workgroups until the chip
     // has ~8 waves per SIMD, at least 32 keys per share
     long splits = 8192 / std::max<long>(1, (long)Tn * H);
-    splits = std::min<long>({splits, 16, (window + 31) / 32});
+    splits = std::min<long>({splits, 16, (reach + 31) / 32});
     splits = std::max<long>(splits, 1);
     if (splits > 1) alloc_parts(splits);
     const int rc = launch_latent_attn(
@@ -318,7 +331,7 @@ Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
         block_table.data_ptr<int>(), (int)block_table.size(1),
         positions.data_ptr<int>(), seq_idx.data_ptr<int>(), out.data_ptr(),
         pa, pm, (int)splits, Tn, H, C, R, (int)cache.size(1), (int)window,
-        (float)scale, c, stream());
+        (float)scale, c, sk, stream());
     TORCH_CHECK(rc == 0, "latent_attn: kv_rank + rot_dim must be <= 1024");
     return out;
 }
@@ -641,7 +654,8 @@ void sink_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
                const Tensor& block_table, const Tensor& positions,
                const Tensor& seq_idx, const Tensor& cu,
                const std::optional<Tensor>& sink, int64_t window, Tensor& out,
-               double out_scale, int64_t max_qlen) {
+               double out_scale, int64_t max_qlen,
+               const std::optional<Tensor>& head_gate) {
     const int c = act_code(q, "q");
     check_i32(block_table, "block_table");
     check_i32(positions, "positions");
@@ -668,13 +682,20 @@ void sink_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
         sk = sink->data_ptr<float>();
     }
     check_i32(cu, "cu_seqlens");
+    const void* hg = nullptr;
+    long hg_tok = 0;
+    if (head_gate.has_value()) {
+        // raw gate, one number per (token, head), a column slice
+        check_slice(*head_gate, Tn, H, q.scalar_type(), "head_gate");
+        hg = head_gate->data_ptr();
+        hg_tok = head_gate->stride(0);
+    }
     // bf16 prompt portions with head size 64/128 run on the matrix cores
     // (the dense models' paged prefill kernel, with the weights as a bf16
-    // pair and the sink in its epilogue); single rows in the same step ride
-    // along. fp32, other head sizes, windows and pure decode steps take the
-    // generic kernel below.
-    if (c == 0 && max_qlen >= 16 && window == 0 && D == Dv &&
-        (D == 64 || D == 128)) {
+    // pair, window-aware tile skipping, and the sink and head gate in its
+    // epilogue); single rows in the same step ride along. fp32, other head
+    // sizes and pure decode steps take the generic kernel below.
+    if (c == 0 && max_qlen >= 16 && D == Dv && (D == 64 || D == 128)) {
         const long B = cu.numel() - 1;
         TORCH_CHECK(block_table.size(0) == B);
         Tensor last = cu.slice(0, 1, B + 1).to(torch::kLong) - 1;
@@ -688,7 +709,8 @@ void sink_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
             block_table.data_ptr<int>(), seq_lens.data_ptr<int>(),
             (unsigned short*)out.data_ptr(), out.stride(0), (int)B, H, G, D,
             (int)block_table.size(1), bs, (int)max_qlen, sk,
-            (float)out_scale, stream());
+            (float)out_scale, (int)window, (const unsigned short*)hg, hg_tok,
+            stream());
         TORCH_CHECK(rc == 0, "sink_attn: matrix-core path refused a shape "
                              "its guard admitted");
         return;
@@ -716,7 +738,7 @@ void sink_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
         block_table.data_ptr<int>(), (int)block_table.size(1),
         positions.data_ptr<int>(), seq_idx.data_ptr<int>(), sk,
         out.data_ptr(), out.stride(0), (float)out_scale, pa, pm, (int)splits,
-        Tn, H, G, D, Dv, bs, (int)window, c, stream());
+        Tn, H, G, D, Dv, bs, (int)window, c, hg, hg_tok, stream());
     TORCH_CHECK(rc == 0, "sink_attn: head sizes must be <= 256");
 }
 
@@ -732,7 +754,13 @@ void register_hybrid_ops(pybind11::module_& m) {
     m.def("latent_rope_store", &latent_rope_store,
           "latent norm + rotation + paged store; q rotation in place");
     m.def("latent_attn", &latent_attn,
-          "windowed attention over the paged latent cache (absorbed form)");
+          "windowed attention over the paged latent cache (absorbed form)",
+          pybind11::arg("q_abs"), pybind11::arg("q_rot"),
+          pybind11::arg("gate"), pybind11::arg("cache"),
+          pybind11::arg("block_table"), pybind11::arg("positions"),
+          pybind11::arg("seq_idx"), pybind11::arg("cu_seqlens"),
+          pybind11::arg("window"), pybind11::arg("scale"),
+          pybind11::arg("max_qlen"), pybind11::arg("sink") = std::nullopt);
     m.def("lightning_attn", &lightning_attn,
           "decayed linear attention with carried fp32 state");
     m.def("retention_attn", &retention_attn,
@@ -751,5 +779,12 @@ void register_hybrid_ops(pybind11::module_& m) {
     m.def("qk_norm_rope_store", &qk_norm_rope_store,
           "q/k head norm + rotation; keys and raw keys to the pages");
     m.def("sink_attn", &sink_attn,
-          "paged causal GQA softmax attention with a sink logit");
+          "paged causal GQA softmax attention with a sink logit",
+          pybind11::arg("q"), pybind11::arg("k_cache"),
+          pybind11::arg("v_cache"), pybind11::arg("block_table"),
+          pybind11::arg("positions"), pybind11::arg("seq_idx"),
+          pybind11::arg("cu_seqlens"), pybind11::arg("sink"),
+          pybind11::arg("window"), pybind11::arg("out"),
+          pybind11::arg("out_scale"), pybind11::arg("max_qlen"),
+          pybind11::arg("head_gate") = std::nullopt);
 }

@@ -49,7 +49,7 @@ latent_attn_kernel(const T* __restrict__ q_abs,   // [H, Tn, C]
                    float* __restrict__ part_acc,  // [splits, H, Tn, C]
                    float* __restrict__ part_ml,   // [splits, H, Tn, 2]
                    int Tn, int H, int C, int R, int bs, int window,
-                   float scale) {
+                   float scale, const float* __restrict__ sink) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x % WAVE;
     const int h = blockIdx.y * LA_WAVES + threadIdx.x / WAVE;
@@ -139,7 +139,14 @@ latent_attn_kernel(const T* __restrict__ q_abs,   // [H, Tn, C]
         return;
     }
     const float g = 1.f / (1.f + expf(-ldf(gate + (long)t * gate_tok + h)));
-    const float r = g / l;
+    float r = g / l;
+    if (sink) {
+        // a logit that joins the denominator without key or value
+        const float sk = sink[h];
+        const float M = fmaxf(m, sk);
+        const float w = expf(m - M);
+        r = g * w / (l * w + expf(sk - M));
+    }
     T* o = out + ((long)h * Tn + t) * C;
 #pragma unroll
     for (int j = 0; j < DPL; ++j) {
@@ -176,7 +183,8 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
                         unsigned short* __restrict__ out,
                         float* __restrict__ part_acc,
                         float* __restrict__ part_ml, int Tn, int H, int C,
-                        int R, int bs, int window, float scale) {
+                        int R, int bs, int window, float scale,
+                        const float* __restrict__ sink) {
     constexpr int DKP = KSTEPS * 32;
     constexpr int KS = DKP + LM_PAD;       // key tile row stride
     constexpr int PS = LM_TN + LM_PAD;     // weight tile row stride
@@ -366,7 +374,13 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
             } else {
                 const float g = 1.f / (1.f + expf(-bf2f(
                     gate[(long)s0 * gate_tok + hh])));
-                const float inv = l_run[r] > 0.f ? g / l_run[r] : 0.f;
+                float inv = l_run[r] > 0.f ? g / l_run[r] : 0.f;
+                if (sink) {
+                    const float sk = sink[hh];
+                    const float M = fmaxf(m_run[r], sk);
+                    const float w = expf(m_run[r] - M);
+                    inv = g * w / (l_run[r] * w + expf(sk - M));
+                }
                 unsigned short* orow = out + ((long)hh * Tn + s0) * C;
 #pragma unroll
                 for (int j = 0; j < NBW; ++j) {
@@ -384,7 +398,13 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
         if (qrow >= QL) continue;
         const float g = 1.f / (1.f + expf(-bf2f(
             gate[(long)(s0 + qrow) * gate_tok + h])));
-        const float inv = l_run[r] > 0.f ? g / l_run[r] : 0.f;
+        float inv = l_run[r] > 0.f ? g / l_run[r] : 0.f;
+        if (sink) {
+            const float sk = sink[h];
+            const float M = fmaxf(m_run[r], sk);
+            const float w = expf(m_run[r] - M);
+            inv = g * w / (l_run[r] * w + expf(sk - M));
+        }
         unsigned short* orow = out + ((long)h * Tn + s0 + qrow) * C;
 #pragma unroll
         for (int j = 0; j < NBW; ++j) {
@@ -406,7 +426,7 @@ latent_attn_combine_kernel(const float* __restrict__ part_acc,
                            const float* __restrict__ part_ml,
                            const T* __restrict__ gate, long gate_tok,
                            T* __restrict__ out, int splits, int Tn, int H,
-                           int C) {
+                           int C, const float* __restrict__ sink) {
     const int t = blockIdx.x, h = blockIdx.y;
     const int lane = threadIdx.x % WAVE;
     float m = -INFINITY, l = 0.f;
@@ -415,9 +435,11 @@ latent_attn_combine_kernel(const float* __restrict__ part_acc,
         m = part_ml[row * 2];
         l = part_ml[row * 2 + 1];
     }
-    const float M = wave_max(l > 0.f ? m : -INFINITY);
+    float M = wave_max(l > 0.f ? m : -INFINITY);
+    if (sink) M = fmaxf(M, sink[h]);
     const float w = l > 0.f ? expf(m - M) : 0.f;
-    const float L = wave_sum(l * w);
+    float L = wave_sum(l * w);
+    if (sink) L += expf(sink[h] - M);
     const float g = 1.f / (1.f + expf(-ldf(gate + (long)t * gate_tok + h)));
     const float r = g / L;
     T* o = out + ((long)h * Tn + t) * C;
@@ -989,7 +1011,8 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
                  const float* __restrict__ sink, T* __restrict__ out,
                  long out_tok, float out_scale, float* __restrict__ part_acc,
                  float* __restrict__ part_ml, int Tn, int H, int G, int D,
-                 int Dv, int bs, int window) {
+                 int Dv, int bs, int window,
+                 const T* __restrict__ head_gate, long hg_tok) {
     extern __shared__ __attribute__((aligned(16))) float sa_q[];
     const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const int t = blockIdx.x;
@@ -1085,7 +1108,9 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
                 w = expf(m[r] - M);
                 L = l[r] * w + expf(sk - M);
             }
-            const float rcp = L > 0.f ? out_scale * w / L : 0.f;
+            float rcp = L > 0.f ? out_scale * w / L : 0.f;
+            if (head_gate)      // sigmoid gate, one number per (token, head)
+                rcp /= 1.f + expf(-ldf(head_gate + (long)t * hg_tok + h));
             T* o = out + (long)t * out_tok + (long)h * Dv;
 #pragma unroll
             for (int i = 0; i < DPL; ++i) {
@@ -1114,7 +1139,8 @@ sink_attn_combine_kernel(const float* __restrict__ part_acc,
                          const float* __restrict__ part_ml,
                          const float* __restrict__ sink, T* __restrict__ out,
                          long out_tok, float out_scale, int splits, int Tn,
-                         int H, int Dv) {
+                         int H, int Dv, const T* __restrict__ head_gate,
+                         long hg_tok) {
     const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const int t = blockIdx.x, h = blockIdx.y * SA_WAVES + wid;
     if (h >= H) return;
@@ -1129,7 +1155,9 @@ sink_attn_combine_kernel(const float* __restrict__ part_acc,
     const float w = l > 0.f ? expf(m - M) : 0.f;
     float L = wave_sum(l * w);
     if (sink) L += expf(sink[h] - M);
-    const float rcp = L > 0.f ? out_scale / L : 0.f;
+    float rcp = L > 0.f ? out_scale / L : 0.f;
+    if (head_gate)
+        rcp /= 1.f + expf(-ldf(head_gate + (long)t * hg_tok + h));
     T* o = out + (long)t * out_tok + (long)h * Dv;
     for (int d0 = 0; d0 < Dv; d0 += WAVE) {
         const int d = d0 + lane;
@@ -1160,7 +1188,7 @@ sink_attn_combine_kernel(const float* __restrict__ part_acc,
             (const TT*)q_abs, (const TT*)q_rot, qr_tok, qr_head,              \
             (const TT*)gate, gate_tok, (const TT*)cache, block_table,         \
             bt_stride, positions, seq_idx, (TT*)out, part_acc, part_ml, Tn,   \
-            H, C, R, bs, window, scale);                                      \
+            H, C, R, bs, window, scale, sink);                                \
         break;
 
 template <typename TT>
@@ -1172,7 +1200,7 @@ static int latent_attn_dispatch(const void* q_abs, const void* q_rot,
                                 void* out, float* part_acc, float* part_ml,
                                 int splits, int Tn, int H, int C, int R,
                                 int bs, int window, float scale,
-                                hipStream_t s) {
+                                const float* sink, hipStream_t s) {
     const int need = (C + R + WAVE - 1) / WAVE;
     const int sizes[] = {1, 2, 3, 4, 6, 9, 12, 16};
     int dpl = 0;
@@ -1188,7 +1216,7 @@ static int latent_attn_dispatch(const void* q_abs, const void* q_rot,
         const dim3 g2(Tn, H);
         latent_attn_combine_kernel<TT><<<g2, LC_THREADS, 0, s>>>(
             part_acc, part_ml, (const TT*)gate, gate_tok, (TT*)out, splits,
-            Tn, H, C);
+            Tn, H, C, sink);
     }
     return 0;
 }
@@ -1202,17 +1230,17 @@ extern "C" int launch_latent_attn(const void* q_abs, const void* q_rot,
                                   void* out, float* part_acc, float* part_ml,
                                   int splits, int Tn, int H, int C, int R,
                                   int bs, int window, float scale, int f32,
-                                  hipStream_t s) {
+                                  const float* sink, hipStream_t s) {
     if (Tn == 0) return 0;
     if (f32)
         return latent_attn_dispatch<float>(
             q_abs, q_rot, qr_tok, qr_head, gate, gate_tok, cache, block_table,
             bt_stride, positions, seq_idx, out, part_acc, part_ml, splits, Tn,
-            H, C, R, bs, window, scale, s);
+            H, C, R, bs, window, scale, sink, s);
     return latent_attn_dispatch<unsigned short>(
         q_abs, q_rot, qr_tok, qr_head, gate, gate_tok, cache, block_table,
         bt_stride, positions, seq_idx, out, part_acc, part_ml, splits, Tn, H,
-        C, R, bs, window, scale, s);
+        C, R, bs, window, scale, sink, s);
 }
 
 #define LM_CASE(N, DEC, TH)                                                   \
@@ -1221,7 +1249,7 @@ extern "C" int launch_latent_attn(const void* q_abs, const void* q_rot,
         qr_head, (const unsigned short*)gate, gate_tok,                       \
         (const unsigned short*)cache, block_table, bt_stride, cu, positions,  \
         seq_idx, (unsigned short*)out, part_acc, part_ml, Tn, H, C, R, bs,    \
-        window, scale)
+        window, scale, sink)
 
 // bf16 on the matrix cores: prompt portions (max_qlen >= 16; 16-query x
 // 4-head workgroups over B sequences) or pure decode steps (max_qlen == 1;
@@ -1235,7 +1263,8 @@ extern "C" int launch_latent_attn_mfma(
     const int* block_table, int bt_stride, const int* cu,
     const int* positions, const int* seq_idx, void* out, float* part_acc,
     float* part_ml, int splits, int Tn, int B, int max_qlen, int H, int C,
-    int R, int bs, int window, float scale, hipStream_t s) {
+    int R, int bs, int window, float scale, const float* sink,
+    hipStream_t s) {
     const int Dk = C + R;
     if (C % 8 != 0 || R % 8 != 0 || Dk > 576) return 1;
     if (Tn == 0 || B == 0) return 0;
@@ -1251,7 +1280,7 @@ extern "C" int launch_latent_attn_mfma(
             latent_attn_combine_kernel<unsigned short>
                 <<<g2, LC_THREADS, 0, s>>>(
                     part_acc, part_ml, (const unsigned short*)gate, gate_tok,
-                    (unsigned short*)out, splits, Tn, H, C);
+                    (unsigned short*)out, splits, Tn, H, C, sink);
         }
         return 0;
     }
@@ -1375,7 +1404,8 @@ extern "C" int launch_delta_rule(const float* q, const float* k, long qk_tok,
     sink_attn_kernel<TT, N, R, P><<<grid, SA_WAVES * WAVE, smem, s>>>(        \
         (const TT*)q, q_tok, (const TT*)k_cache, (const TT*)v_cache,          \
         block_table, bt_stride, positions, seq_idx, sink, (TT*)out, out_tok,  \
-        out_scale, part_acc, part_ml, Tn, H, G, D, Dv, bs, window)
+        out_scale, part_acc, part_ml, Tn, H, G, D, Dv, bs, window,            \
+        (const TT*)head_gate, hg_tok)
 
 #define SA_CASE(N, P)                                                         \
     if (dpl == N && pair == P) {                                              \
@@ -1393,7 +1423,8 @@ static int sink_attn_dispatch(const void* q, long q_tok, const void* k_cache,
                               void* out, long out_tok, float out_scale,
                               float* part_acc, float* part_ml, int splits,
                               int Tn, int H, int G, int D, int Dv, int bs,
-                              int window, hipStream_t s) {
+                              int window, const void* head_gate, long hg_tok,
+                              hipStream_t s) {
     // even value sizes: a lane owns coordinate pairs (one load for two)
     const bool pair = Dv % 2 == 0;
     int dpl = pair ? 2 * ((Dv + 2 * WAVE - 1) / (2 * WAVE))
@@ -1413,12 +1444,14 @@ static int sink_attn_dispatch(const void* q, long q_tok, const void* k_cache,
         const dim3 g2(Tn, (H + SA_WAVES - 1) / SA_WAVES);
         sink_attn_combine_kernel<TT><<<g2, SA_WAVES * WAVE, 0, s>>>(
             part_acc, part_ml, sink, (TT*)out, out_tok, out_scale, splits, Tn,
-            H, Dv);
+            H, Dv, (const TT*)head_gate, hg_tok);
     }
     return 0;
 }
 
-// returns nonzero when a head size exceeds 256
+// head_gate (optional, activation type, [Tn, H] with row stride hg_tok):
+// head h's output times sigmoid(head_gate[t, h]). Returns nonzero when a
+// head size exceeds 256.
 extern "C" int launch_sink_attn(const void* q, long q_tok,
                                 const void* k_cache, const void* v_cache,
                                 const int* block_table, int bt_stride,
@@ -1427,18 +1460,19 @@ extern "C" int launch_sink_attn(const void* q, long q_tok,
                                 float out_scale, float* part_acc,
                                 float* part_ml, int splits, int Tn, int H,
                                 int G, int D, int Dv, int bs, int window,
-                                int f32, hipStream_t s) {
+                                int f32, const void* head_gate, long hg_tok,
+                                hipStream_t s) {
     if (D > SA_MAXD || Dv > SA_MAXD) return 1;
     if (Tn == 0) return 0;
     if (f32)
         return sink_attn_dispatch<float>(
             q, q_tok, k_cache, v_cache, block_table, bt_stride, positions,
             seq_idx, sink, out, out_tok, out_scale, part_acc, part_ml, splits,
-            Tn, H, G, D, Dv, bs, window, s);
+            Tn, H, G, D, Dv, bs, window, head_gate, hg_tok, s);
     return sink_attn_dispatch<unsigned short>(
         q, q_tok, k_cache, v_cache, block_table, bt_stride, positions,
         seq_idx, sink, out, out_tok, out_scale, part_acc, part_ml, splits, Tn,
-        H, G, D, Dv, bs, window, s);
+        H, G, D, Dv, bs, window, head_gate, hg_tok, s);
 }
 
 // ---------------------------------------------------------------------------
@@ -1670,7 +1704,7 @@ talk_scores_kernel(const T* __restrict__ q, long q_tok,
                    const int* __restrict__ seq_idx,
                    float* __restrict__ scores, long ctx,
                    float* __restrict__ part_ml, int Tn, int H, int G, int D,
-                   int bs, int window) {
+                   int bs, int window, float softcap) {
     extern __shared__ __attribute__((aligned(16))) float sa_q[];
     const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const int t = blockIdx.x;
@@ -1707,6 +1741,8 @@ talk_scores_kernel(const T* __restrict__ q, long q_tok,
         }
 #pragma unroll
         for (int r = 0; r < REP; ++r) {
+            // softcap > 0: the stored score is softcap * tanh(s / softcap)
+            if (softcap > 0.f) sc[r] = softcap * tanhf(sc[r] / softcap);
             const float sv = valid ? sc[r] : -INFINITY;
             if (valid)
                 scores[((long)t * H + h0 + r) * ctx + (j - lo)] = sv;
@@ -1907,7 +1943,8 @@ static int talk_scored_dispatch(const void* q, long q_tok, const void* k_cache,
 #define TS_LAUNCH(R)                                                          \
     talk_scores_kernel<TT, R><<<grid, SA_WAVES * WAVE, smem1, s>>>(           \
         (const TT*)q, q_tok, (const TT*)k_cache, block_table, bt_stride,      \
-        positions, seq_idx, scores, ctx, part_ml, Tn, H, G, D, bs, window)
+        positions, seq_idx, scores, ctx, part_ml, Tn, H, G, D, bs, window,    \
+        0.f)
     if (rep == 4) TS_LAUNCH(4);
     else if (rep == 2) TS_LAUNCH(2);
     else TS_LAUNCH(1);
@@ -2037,4 +2074,244 @@ extern "C" int launch_talk_mix(const float* part_acc, const float* part_ml,
             part_acc, part_ml, talk, (const unsigned short*)gate, gate_tok,
             (unsigned short*)out, out_tok, splits, Tn, H, G, Dv);
     return 0;
+}
+
+
+// ---------------------------------------------------------------------------
+// mixed_score_attn: windowed grouped-query softmax attention whose (capped)
+// scores are mixed across heads BEFORE the softmax,
+//   s'_h(j) = sum_g mix[h, g] s_g(j),   o_h = softmax_j(s'_h) v_{c(h)}(j),
+// c(h) the key/value head of query head h. Kernel 1 (talk_scores_kernel
+// with its cap) writes every head's score of every visible key once; kernel
+// 2 below reads, per key, the scores of ALL heads, mixes them with the
+// wave's rows of `mix`, and runs sink_attn's online softmax and value sum on
+// the mixed scores: wave = (token, REP query heads of one key group, key
+// split), lane = key for the scores, lane = coordinate pair for the value
+// sum, each cached value row read once per key group. Partials and the merge
+// are sink_attn's (sink_attn_combine_kernel), so an optional sink logit and
+// a per-head sigmoid gate come with it.
+namespace {
+
+template <typename T, int DPL, int REP, bool PAIR>
+__global__ void __launch_bounds__(SA_WAVES * WAVE)
+mixed_score_pv_kernel(const float* __restrict__ scores, long ctx,
+                      const float* __restrict__ mix,
+                      const T* __restrict__ v_cache,
+                      const int* __restrict__ block_table, int bt_stride,
+                      const int* __restrict__ positions,
+                      const int* __restrict__ seq_idx,
+                      const float* __restrict__ sink, T* __restrict__ out,
+                      long out_tok, float* __restrict__ part_acc,
+                      float* __restrict__ part_ml, int Tn, int H, int G,
+                      int Dv, int bs, int window,
+                      const T* __restrict__ head_gate, long hg_tok) {
+    extern __shared__ __attribute__((aligned(16))) float ms_s[];
+    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int t = blockIdx.x;
+    const int unit = blockIdx.y * SA_WAVES + wid;
+    if (unit * REP >= H) return;      // no workgroup barrier below
+    const int h0 = unit * REP;
+    const int split = blockIdx.z, nsplit = gridDim.z;
+    const int p = positions[t];
+    const int g = h0 / (H / G);
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int per =
+        ((p + 1 - lo + nsplit - 1) / nsplit + WAVE - 1) / WAVE * WAVE;
+    const int klo = lo + split * per, khi = min(p + 1, klo + per);
+    float* mw = ms_s + (long)wid * REP * H;         // the wave's rows of mix
+    for (int i = lane; i < REP * H; i += WAVE) mw[i] = mix[(long)h0 * H + i];
+    WAVE_LDS_SYNC();
+    const int* bt = block_table + (long)seq_idx[t] * bt_stride;
+    const float* srow = scores + (long)t * H * ctx;
+    float m[REP], l[REP], acc[REP][DPL];
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+        m[r] = -INFINITY;
+        l[r] = 0.f;
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) acc[r][i] = 0.f;
+    }
+    for (int j0 = klo; j0 < khi; j0 += WAVE) {
+        const int j = j0 + lane;
+        const bool valid = j < khi;
+        const int nk = min(WAVE, khi - j0);
+        int row = 0;            // lanes past the end point at a real row
+        float sc[REP], pj[REP];
+#pragma unroll
+        for (int r = 0; r < REP; ++r) sc[r] = 0.f;
+        if (valid) {
+            row = (bt[j / bs] * G + g) * bs + j % bs;
+            for (int gq = 0; gq < H; ++gq) {
+                const float sv = srow[(long)gq * ctx + (j - lo)];
+#pragma unroll
+                for (int r = 0; r < REP; ++r) sc[r] += mw[r * H + gq] * sv;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < REP; ++r) {
+            const float sv = valid ? sc[r] : -INFINITY;
+            const float m_new = fmaxf(m[r], wave_max(sv));
+            pj[r] = valid ? expf(sv - m_new) : 0.f;
+            const float corr = expf(m[r] - m_new);
+            l[r] = l[r] * corr + wave_sum(pj[r]);
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) acc[r][i] *= corr;
+            m[r] = m_new;
+        }
+#pragma unroll 2
+        for (int jj = 0; jj < nk; jj += SA_PV) {
+            float vv[SA_PV][DPL];
+#pragma unroll
+            for (int u = 0; u < SA_PV; ++u) {
+                const T* vr =
+                    v_cache + (long)__builtin_amdgcn_readlane(row, jj + u) * Dv;
+                if constexpr (PAIR) {
+#pragma unroll
+                    for (int i = 0; i < DPL; i += 2) {
+                        const int d = sa_coord<true>(lane, i);
+                        vv[u][i] = vv[u][i + 1] = 0.f;
+                        if (d < Dv) sa_ld2(vr + d, vv[u][i], vv[u][i + 1]);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < DPL; ++i) {
+                        const int d = sa_coord<false>(lane, i);
+                        vv[u][i] = d < Dv ? ldf(vr + d) : 0.f;
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < SA_PV; ++u)
+#pragma unroll
+                for (int r = 0; r < REP; ++r) {
+                    const float pb = __builtin_bit_cast(
+                        float, __builtin_amdgcn_readlane(
+                                   __builtin_bit_cast(int, pj[r]), jj + u));
+#pragma unroll
+                    for (int i = 0; i < DPL; ++i) acc[r][i] += pb * vv[u][i];
+                }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+        const int h = h0 + r;
+        if (nsplit == 1) {
+            float L = l[r], w = 1.f;
+            if (sink) {
+                const float sk = sink[h];
+                const float M = fmaxf(m[r], sk);
+                w = expf(m[r] - M);
+                L = l[r] * w + expf(sk - M);
+            }
+            float rcp = L > 0.f ? w / L : 0.f;
+            if (head_gate)
+                rcp /= 1.f + expf(-ldf(head_gate + (long)t * hg_tok + h));
+            T* o = out + (long)t * out_tok + (long)h * Dv;
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) {
+                const int d = sa_coord<PAIR>(lane, i);
+                if (d < Dv) stf(o + d, acc[r][i] * rcp);
+            }
+        } else {
+            const long prow = ((long)split * H + h) * Tn + t;
+            if (lane == 0) {
+                part_ml[prow * 2] = m[r];
+                part_ml[prow * 2 + 1] = l[r];
+            }
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) {
+                const int d = sa_coord<PAIR>(lane, i);
+                if (d < Dv) part_acc[prow * Dv + d] = acc[r][i];
+            }
+        }
+    }
+}
+
+}  // namespace
+
+#define MS_LAUNCH(N, R, P)                                                    \
+    mixed_score_pv_kernel<TT, N, R, P>                                        \
+        <<<grid, SA_WAVES * WAVE, smem2, s>>>(                                \
+            scores, ctx, mix, (const TT*)v_cache, block_table, bt_stride,     \
+            positions, seq_idx, sink, (TT*)out, out_tok, part_acc, part_ml,   \
+            Tn, H, G, Dv, bs, window, (const TT*)head_gate, hg_tok)
+
+#define MS_CASE(N, P)                                                         \
+    if (dpl == N && pair == P) {                                              \
+        if (rep == 4) MS_LAUNCH(N, 4, P);                                     \
+        else if (rep == 2) MS_LAUNCH(N, 2, P);                                \
+        else MS_LAUNCH(N, 1, P);                                              \
+        launched = true;                                                      \
+    }
+
+template <typename TT>
+static int mixed_score_dispatch(const void* q, long q_tok, const void* k_cache,
+                                const void* v_cache, const int* block_table,
+                                int bt_stride, const int* positions,
+                                const int* seq_idx, float softcap,
+                                const float* mix, const float* sink,
+                                const void* head_gate, long hg_tok, void* out,
+                                long out_tok, float* scores, long ctx,
+                                float* scratch_ml, float* part_acc,
+                                float* part_ml, int splits, int Tn, int H,
+                                int G, int D, int Dv, int bs, int window,
+                                hipStream_t s) {
+    const bool pair = Dv % 2 == 0;
+    int dpl = pair ? 2 * ((Dv + 2 * WAVE - 1) / (2 * WAVE))
+                   : (Dv + WAVE - 1) / WAVE;
+    if (dpl == 3) dpl = 4;
+    const int group = H / G;
+    const int rep = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
+    const int units = H / rep;
+    const dim3 grid(Tn, (units + SA_WAVES - 1) / SA_WAVES, splits);
+    const size_t smem1 = (size_t)SA_WAVES * rep * D * sizeof(float);
+    const size_t smem2 = (size_t)SA_WAVES * rep * H * sizeof(float);
+#define TS_LAUNCH(R)                                                          \
+    talk_scores_kernel<TT, R><<<grid, SA_WAVES * WAVE, smem1, s>>>(           \
+        (const TT*)q, q_tok, (const TT*)k_cache, block_table, bt_stride,      \
+        positions, seq_idx, scores, ctx, scratch_ml, Tn, H, G, D, bs, window, \
+        softcap)
+    if (rep == 4) TS_LAUNCH(4);
+    else if (rep == 2) TS_LAUNCH(2);
+    else TS_LAUNCH(1);
+#undef TS_LAUNCH
+    bool launched = false;
+    MS_CASE(2, true) MS_CASE(4, true)
+    MS_CASE(1, false) MS_CASE(2, false) MS_CASE(4, false)
+    if (!launched) return 1;
+    if (splits > 1) {
+        const dim3 g2(Tn, (H + SA_WAVES - 1) / SA_WAVES);
+        sink_attn_combine_kernel<TT><<<g2, SA_WAVES * WAVE, 0, s>>>(
+            part_acc, part_ml, sink, (TT*)out, out_tok, 1.f, splits, Tn, H, Dv,
+            (const TT*)head_gate, hg_tok);
+    }
+    return 0;
+}
+
+// scores [Tn, H, ctx] fp32 (ctx >= the longest visible key range);
+// scratch_ml [splits, Tn, H, 2] (per-split statistics of the unmixed scores,
+// unused); part_acc [splits, H, Tn, Dv], part_ml [splits, H, Tn, 2] (unused
+// when splits == 1). mix fp32 [H, H]; softcap 0: no cap. Nonzero when a head
+// size exceeds 256.
+extern "C" int launch_mixed_score_attn(
+    const void* q, long q_tok, const void* k_cache, const void* v_cache,
+    const int* block_table, int bt_stride, const int* positions,
+    const int* seq_idx, float softcap, const float* mix, const float* sink,
+    const void* head_gate, long hg_tok, void* out, long out_tok, float* scores,
+    long ctx, float* scratch_ml, float* part_acc, float* part_ml, int splits,
+    int Tn, int H, int G, int D, int Dv, int bs, int window, int f32,
+    hipStream_t s) {
+    if (D > SA_MAXD || Dv > SA_MAXD) return 1;
+    if (Tn == 0) return 0;
+    if (f32)
+        return mixed_score_dispatch<float>(
+            q, q_tok, k_cache, v_cache, block_table, bt_stride, positions,
+            seq_idx, softcap, mix, sink, head_gate, hg_tok, out, out_tok,
+            scores, ctx, scratch_ml, part_acc, part_ml, splits, Tn, H, G, D,
+            Dv, bs, window, s);
+    return mixed_score_dispatch<unsigned short>(
+        q, q_tok, k_cache, v_cache, block_table, bt_stride, positions,
+        seq_idx, softcap, mix, sink, head_gate, hg_tok, out, out_tok, scores,
+        ctx, scratch_ml, part_acc, part_ml, splits, Tn, H, G, D, Dv, bs,
+        window, s);
 }

@@ -29,6 +29,8 @@ ext = CUDAExtension(
         os.path.join(CSRC, "mixers.hip"),
         os.path.join(CSRC, "sandwich_ext.cpp"),
         os.path.join(CSRC, "sandwich.hip"),
+        os.path.join(CSRC, "gated_ext.cpp"),
+        os.path.join(CSRC, "gated.hip"),
     ],
     extra_compile_args={
         "cxx": ["-O3", "-std=c++17"]
