@@ -730,8 +730,11 @@ class Runner:
         off = cols(pre + "q")
         qkv = off.as_strided((T, nq + nk + nv), off.stride())
         if ns.conv_w is not None:
-            qkv = ops.short_conv(qkv, ns.conv_w, self.kv.conv_state[i],
-                                 state_slots, cu, seq_idx, positions, False)
+            conv_state = self.kv.conv_state[i]
+            if conv_state is None:       # a single tap carries nothing
+                conv_state = qkv.new_empty(0)
+            qkv = ops.short_conv(qkv, ns.conv_w, conv_state, state_slots, cu,
+                                 seq_idx, positions, False)
         q = qkv[:, :nq].view(T, m.heads, m.dim)
         k = qkv[:, nq : nq + nk].view(T, m.kv_heads, m.dim)
         v = qkv[:, nq + nk :].view(T, m.kv_heads, m.vdim)

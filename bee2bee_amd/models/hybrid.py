@@ -957,18 +957,17 @@ def pimodra_layers(n_layers: int, width: int, *, heads: int = 16,
     return looped_layer_specs_from_cfg(cfg_layers, lp)
 
 
-def zevilorn_layers(n_layers: int, width: int, *, heads: int = 16,
-                    kv_heads: int = 4, dim: int = 128, window: int = 1024,
-                    kv_rank: int = 512, rot_dim: int = 64, q_rank: int = 768,
-                    gru_width: Optional[int] = None, experts: int = 8,
-                    top_k: int = 2, expert_ff: int = 1024, groups: int = 4,
-                    keep: int = 2, taps: int = 4,
-                    loop: Optional[Tuple[int, int, int]] = None
-                    ) -> List[LayerSpec]:
-    """A synthetic Zevilorn stack for benchmarks: the cycle capped
-    score-mixing attention / latent attention / windowed attention beside a
-    minGRU, every layer with group-routed gelu experts; loop = (start,
-    stop, times) repeats a block with shared tensors."""
+def zevilorn_layer_cfgs(n_layers: int, width: int, *, heads: int = 16,
+                        kv_heads: int = 4, dim: int = 128, window: int = 1024,
+                        kv_rank: int = 512, rot_dim: int = 64,
+                        q_rank: int = 768, gru_width: Optional[int] = None,
+                        experts: int = 8, top_k: int = 2,
+                        expert_ff: int = 1024, groups: int = 4, keep: int = 2,
+                        taps: int = 4) -> List[Dict[str, Any]]:
+    """config.json 'layers' entries of a synthetic Zevilorn stack for
+    benchmarks: the cycle capped score-mixing attention / latent attention
+    / windowed attention beside a minGRU, every layer with group-routed
+    gelu experts."""
     cfg_layers = []
     mlp = {"kind": "moe", "expert": {"ff": expert_ff},
            "router": {"experts": experts, "top": top_k,
@@ -999,7 +998,4 @@ def zevilorn_layers(n_layers: int, width: int, *, heads: int = 16,
                                       "scaling": {"factor": 2.0}}},
                      "right": {"width": gru_width or width}}
         cfg_layers.append({"type": typ, "mixer": mixer, "mlp": mlp})
-    lp = None
-    if loop:
-        lp = {"start": loop[0], "stop": loop[1], "times": loop[2]}
-    return gated_layer_specs_from_cfg(cfg_layers, lp)
+    return cfg_layers

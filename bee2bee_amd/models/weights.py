@@ -836,16 +836,7 @@ class ModelWeights:
                     # checkpoint [channels, taps] -> tap-major [taps, channels]
                     ns.conv_w = f32(torch.cat(
                         [get(q + "q.conv"), get(q + "k.conv"),
-                         get(q + "v.conv")], dim=0).t()) if m.taps > 1 else None
-                    if m.taps == 1:
-                        # a single tap carries nothing: fold it into the rows
-                        for n_ in ("q", "k", "v"):
-                            off, n = ins[pre + n_]
-                            tap = get(q + n_ + ".conv").to(dev, torch.float32)
-                            w_in[off : off + n] = (
-                                w_in[off : off + n].float() * tap).to(dt)
-                            b_in[off : off + n] = (
-                                b_in[off : off + n].float() * tap[:, 0]).to(dt)
+                         get(q + "v.conv")], dim=0).t()) if m.taps else None
                     ns.talk = f32(get(q + "talk")) if m.score_mix else None
                     ns.wo_b = act(get(q + "o.b")) if m.bias else None
                 elif m.kind == "latent_attention":
@@ -1145,6 +1136,91 @@ def _save_pimodra(weights: "ModelWeights", out_dir: str, tensors, cpu) -> None:
         json.dump(pimodra_config(s), fh, indent=1)
 
 
+def zevilorn_config(spec: ModelSpec) -> Dict:
+    """The config.json dict of a Zevilorn spec (inverse of zevilorn_spec):
+    the layer and loop entries are kept as they were parsed."""
+    src = spec.source_cfg or {}
+    cfg = {"architecture": "Zevilorn", "vocab": spec.vocab_size,
+           "width": spec.hidden_size, "max_seq_len": spec.max_seq_len,
+           "norm": {"eps": spec.rms_eps}, "layers": src.get("layers", [])}
+    if src.get("loop"):
+        cfg["loop"] = dict(src["loop"])
+    return cfg
+
+
+def _save_zevilorn(weights: "ModelWeights", out_dir: str, tensors, cpu) -> None:
+    from safetensors.torch import save_file
+
+    from .hybrid import mixer_parts
+
+    s = weights.spec
+
+    def put(name: str, t: torch.Tensor) -> None:
+        tensors[name] = cpu(t).to(torch.bfloat16)
+
+    put("embed", weights.embed)
+    put("head", weights.lm_head)
+    put("final.norm", weights.final_norm)
+    for i, l in enumerate(s.layer_specs):
+        if l.weights_of is not None:
+            continue
+        lw, p, f = weights.layers[i], f"l{l.src}.", l.ffn
+        ins, _ = lw.layout
+
+        def rows(key: str, name: str, bias: bool = False) -> None:
+            off, n = ins[key]
+            put(name, lw.w_in[off : off + n])
+            if bias:
+                put(name + ".b", lw.b_in[off : off + n])
+
+        put(p + "norm1", lw.norm_w)
+        rows("rg1", p + "rg1", True)
+        for pre, m in mixer_parts(l.mixer):
+            q, ns = p + "mix." + pre, lw.mix[pre]
+            if m.kind == "gqa_attention":
+                off = 0
+                for n_, sz in m.in_sizes:
+                    rows(pre + n_, q + n_, m.bias and n_ != "g")
+                    if ns.conv_w is not None and n_ != "g":
+                        put(q + n_ + ".conv", ns.conv_w[:, off : off + sz].t())
+                        off += sz
+                if ns.talk is not None:
+                    put(q + "talk", ns.talk)
+                if ns.wo_b is not None:
+                    put(q + "o.b", ns.wo_b)
+            elif m.kind == "latent_attention":
+                if m.q_rank:
+                    rows(pre + "dq", q + "dq")
+                    put(q + "dq.norm", ns.q_norm)
+                    put(q + "uq", ns.w_uq)
+                else:
+                    rows(pre + "q", q + "q")
+                rows(pre + "dkv", q + "dkv")
+                rows(pre + "g", q + "g")
+                put(q + "dkv.norm", ns.kv_norm)
+                put(q + "uk", ns.w_uk.reshape(m.heads * m.dim, m.kv_rank))
+                put(q + "uv", ns.w_uv.transpose(1, 2).reshape(
+                    m.heads * m.vdim, m.kv_rank))
+                if ns.sink is not None:
+                    put(q + "sink", ns.sink)
+            else:
+                rows(pre + "z", q + "z", True)
+                rows(pre + "x", q + "x", True)
+                rows(pre + "g", q + "g")
+            put(q + "o", ns.wo)
+            if hasattr(ns, "out_norm"):
+                put(q + "out", ns.out_norm)
+        if f is not None:
+            rows("rg2", p + "rg2", True)
+            put(p + "mlp.router", lw.moe_gate)
+            for e in range(f.n_experts):
+                put(f"{p}mlp.e{e}.up", lw.moe_w_gate_up[e])
+                put(f"{p}mlp.e{e}.down", lw.moe_w_down[e])
+    save_file(tensors, os.path.join(out_dir, "model.safetensors"))
+    with open(os.path.join(out_dir, "config.json"), "w") as fh:
+        json.dump(zevilorn_config(s), fh, indent=1)
+
+
 def safetensors_shapes(model_path: str) -> Dict[str, Tuple[int, ...]]:
     """Tensor name -> shape from the shards' headers (8-byte little-endian
     length, then that many bytes of JSON); no tensor data is read."""
@@ -1438,6 +1514,8 @@ def save_hf(weights: ModelWeights, out_dir: str) -> None:
             _save_pugozen(weights, out_dir, tensors, cpu)
         elif s.arch == "pimodra":
             _save_pimodra(weights, out_dir, tensors, cpu)
+        elif s.arch == "zevilorn":
+            _save_zevilorn(weights, out_dir, tensors, cpu)
         else:
             _save_nukopel(weights, out_dir, tensors, cpu)
         return

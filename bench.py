@@ -217,6 +217,53 @@ def compare_pimodra(args) -> None:
                                     device, p_batch, p_len, d_batch, d_len)
 
 
+def compare_zevilorn(args) -> None:
+    """Prefill and decode throughput of a Zevilorn stack (gated
+    parallel-form layers with an fp32 residual: a grouped-query attention
+    with a short conv on q|k|v, capped scores mixed across heads before the
+    softmax and a zero-logit sink; a latent attention with a normed query
+    latent and a per-head sink; a windowed attention beside a minGRU;
+    group-routed gelu experts in every layer; layers 1-2 of the four run
+    twice with shared tensors) beside the closest stack the framework
+    already served: GQA attention + routed experts at equal width, layer
+    runs, head count/size, key/value heads and expert sizes. The window
+    (4096) covers every context here, so the windowed layers attend the
+    same keys as the dense model. Random weights, synthetic prompts, one
+    GPU."""
+    from bee2bee_amd.models.hybrid import zevilorn_layer_cfgs
+    from bee2bee_amd.models.spec import ModelSpec, zevilorn_spec
+
+    on_gpu = torch.cuda.is_available()
+    device = "cuda:0" if on_gpu else "cpu"
+    vocab, head_dim = 32000, 128
+    p_batch, p_len = 8, (2048 if on_gpu else 48)
+    d_batch, d_len = (64 if on_gpu else 4), (1024 if on_gpu else 32)
+    for size in args.compare_zevilorn.split(","):
+        z = HYBRID_SIZES[size.strip()]
+        W, H, ff, E = z["width"], z["heads"], z["ff"], z["experts"]
+        kv_rank, rot_dim, q_rank = 512, 64, 768
+        if not on_gpu:
+            W, H, head_dim, vocab, ff, E = 64, 4, 16, 256, 32, 4
+            kv_rank, rot_dim, q_rank = 24, 8, 32
+        # 4 checkpoint layers, layers 1..2 run twice: 6 layer runs
+        layers = zevilorn_layer_cfgs(
+            4, W, heads=H, kv_heads=max(1, H // 4), dim=head_dim,
+            window=4096, kv_rank=kv_rank, rot_dim=rot_dim, q_rank=q_rank,
+            gru_width=W, experts=E, top_k=2, expert_ff=ff, groups=4, keep=2)
+        zv = zevilorn_spec(f"zevilorn-{size}", {
+            "vocab": vocab, "width": W, "norm": {"eps": 1e-6},
+            "layers": layers, "max_seq_len": 8192,
+            "loop": {"start": 1, "stop": 3, "times": 2}})
+        dense = ModelSpec(
+            name=f"gqa-moe-{size}", vocab_size=vocab, hidden_size=W,
+            intermediate_size=ff, n_layers=len(zv.layer_specs), n_heads=H,
+            n_kv_heads=max(1, H // 4), head_dim=head_dim, rope_theta=1e6,
+            max_seq_len=8192, n_experts=E, top_k_experts=2)
+        for spec in (zv, dense):
+            _measure_prefill_decode(spec, "zevilorn-vs-dense", size, args,
+                                    device, p_batch, p_len, d_batch, d_len)
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -253,6 +300,16 @@ def main() -> None:
                          "runs, heads and expert sizes, at the "
                          "comma-separated sizes (s, m, l); one JSON line "
                          "per size and model")
+    ap.add_argument("--compare-zevilorn", default=None, metavar="SIZES",
+                    help="instead of the headline run: prefill and decode "
+                         "throughput of the Zevilorn stack (gated "
+                         "parallel-form layers: score-mixing attention, "
+                         "latent attention with a sink, windowed attention "
+                         "beside a minGRU, group-routed gelu experts, a "
+                         "repeated block) beside a GQA-attention MoE stack "
+                         "of equal width, layer runs, heads and expert "
+                         "sizes, at the comma-separated sizes (s, m, l); "
+                         "one JSON line per size and model")
     ap.add_argument("--preflight", action="store_true",
                     help="run the scale-run preflight checks (RCCL self-"
                          "test, master endpoint, env, rank wiring) and exit")
@@ -275,6 +332,9 @@ def main() -> None:
         return
     if args.compare_pimodra:
         compare_pimodra(args)
+        return
+    if args.compare_zevilorn:
+        compare_zevilorn(args)
         return
 
     from bee2bee_amd.models.spec import resolve_spec

@@ -171,7 +171,7 @@ def latent_attention(W, p: str, m: dict, h: torch.Tensor,
     q = linear(W, p + "uq", cq).view(T, H, D + R)
     dkv = linear(W, p + "dkv", h)
     c = unit(dkv[:, :C], eps) * W[p + "dkv.norm"].double()
-    f = frequencies(m["rot"], "none")
+    f = frequencies(dict(m["rot"], scaling=None), "none")
     kr = rotate(dkv[:, C:].reshape(T, 1, R), f, "half")          # [T, 1, R]
     qr = rotate(q[..., D:].contiguous(), f, "half")
     kn = linear(W, p + "uk", c).view(T, H, D)
@@ -310,6 +310,53 @@ def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int],
 
 
 # ------------------------------------------------- random checkpoints
+
+def make_config(vocab=61, width=24, kinds=("attention", "latent_attention",
+                                           "parallel"),
+                loop=(1, 3, 2), heads=4, kv_heads=2, dim=6, vdim=10,
+                window=9, rot_dims=4, scaling=True, softcap=2.5, conv=3,
+                lat_heads=3, lat_dim=6, rot_dim=4, lat_vdim=5, kv_rank=7,
+                q_rank=9, left_heads=4, left_kv=2, left_dim=8, left_vdim=6,
+                left_window=7, left_rot=4, gru=13, experts=8, top=3,
+                n_groups=4, keep=3, ff=10, no_mlp=(), eps=1e-5):
+    """A small config of the design; `kinds` lists the layers, `no_mlp` the
+    indices of layers without a feed-forward, loop = (start, stop, times)."""
+    layers = []
+    for i, kind in enumerate(kinds):
+        if kind == "attention":
+            rot = {"base": 500.0, "dims": rot_dims}
+            if scaling:
+                rot["scaling"] = {"factor": 4.0, "low": 1.0, "high": 4.0,
+                                  "original": 16}
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim,
+                     "vdim": vdim, "scale": dim ** -0.5, "softcap": softcap,
+                     "conv": conv, "mask": {"size": window}}
+            if rot_dims:
+                mixer["rot"] = rot
+        elif kind == "latent_attention":
+            mixer = {"heads": lat_heads, "dim": lat_dim, "rot_dim": rot_dim,
+                     "vdim": lat_vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+                     "scale": (lat_dim + rot_dim) ** -0.5,
+                     "rot": {"base": 300.0, "dims": rot_dim}}
+        else:
+            left = {"heads": left_heads, "kv_heads": left_kv, "dim": left_dim,
+                    "vdim": left_vdim, "scale": left_dim ** -0.5,
+                    "mask": {"size": left_window}}
+            if left_rot:
+                left["rot"] = {"base": 100.0, "dims": left_rot,
+                               "scaling": {"factor": 2.0}}
+            mixer = {"left": left, "right": {"width": gru}}
+        mlp = None if i in no_mlp else {
+            "kind": "moe", "expert": {"ff": ff},
+            "router": {"experts": experts, "top": top,
+                       "groups": {"count": n_groups, "keep": keep}}}
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    cfg = {"architecture": "Zevilorn", "vocab": vocab, "width": width,
+           "norm": {"eps": eps}, "layers": layers}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
 
 def tensor_shapes(cfg: dict) -> Dict[str, tuple]:
     Wd, V = int(cfg["width"]), int(cfg["vocab"])
