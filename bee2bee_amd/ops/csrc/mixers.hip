@@ -1044,12 +1044,14 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
     for (int j0 = klo; j0 < khi; j0 += WAVE) {
         const int j = j0 + lane;
         const bool valid = j < khi;
-        int row = 0;            // lanes past the end point at a real row
+        // lanes past the end point at the share's last key: a row this
+        // sequence wrote (their weights are 0, and 0 x garbage is not 0)
+        const int jc = min(j, khi - 1);
+        const int row = (bt[jc / bs] * G + g) * bs + jc % bs;
         float sc[REP], pj[REP];
 #pragma unroll
         for (int r = 0; r < REP; ++r) sc[r] = 0.f;
         const int nk = min(WAVE, khi - j0);
-        if (valid) row = (bt[j / bs] * G + g) * bs + j % bs;
         if (valid) SaDots<T, REP>::run(k_cache + (long)row * D, qv, D, sc);
 #pragma unroll
         for (int r = 0; r < REP; ++r) {
@@ -1539,7 +1541,10 @@ talk_attn_kernel(const T* __restrict__ q, long q_tok,
 #pragma unroll
         for (int r = 0; r < REP; ++r) sc[r] = 0.f;
         const int nk = min(WAVE, khi - j0);
-        if (valid) row0 = bt[j / bs] * G * bs + j % bs;
+        {   // past the end: the share's last key, a row the sequence wrote
+            const int jc = min(j, khi - 1);
+            row0 = bt[jc / bs] * G * bs + jc % bs;
+        }
         if (valid)
             SaDots<T, REP>::run(k_cache + (long)(row0 + g * bs) * D, qv, D,
                                 sc);
@@ -1821,12 +1826,14 @@ talk_pv_kernel(const float* __restrict__ scores, long ctx,
         const int j = j0 + lane;
         const bool valid = j < khi;
         const int nk = min(WAVE, khi - j0);
-        int row = 0;            // lanes past the end point at a real row
+        // lanes past the end point at the share's last key: a row this
+        // sequence wrote (their weights are 0, and 0 x garbage is not 0)
+        const int jc = min(j, khi - 1);
+        const int row = (bt[jc / bs] * G + g) * bs + jc % bs;
         float pj[REP];
 #pragma unroll
         for (int r = 0; r < REP; ++r) pj[r] = 0.f;
         if (valid) {
-            row = (bt[j / bs] * G + g) * bs + j % bs;
             for (int gq = 0; gq < H; ++gq) {
                 const float e =
                     expf(srow[(long)gq * ctx + (j - lo)] - Mh[gq]) * iL[gq];
@@ -2135,12 +2142,14 @@ mixed_score_pv_kernel(const float* __restrict__ scores, long ctx,
         const int j = j0 + lane;
         const bool valid = j < khi;
         const int nk = min(WAVE, khi - j0);
-        int row = 0;            // lanes past the end point at a real row
+        // lanes past the end point at the share's last key: a row this
+        // sequence wrote (their weights are 0, and 0 x garbage is not 0)
+        const int jc = min(j, khi - 1);
+        const int row = (bt[jc / bs] * G + g) * bs + jc % bs;
         float sc[REP], pj[REP];
 #pragma unroll
         for (int r = 0; r < REP; ++r) sc[r] = 0.f;
         if (valid) {
-            row = (bt[j / bs] * G + g) * bs + j % bs;
             for (int gq = 0; gq < H; ++gq) {
                 const float sv = srow[(long)gq * ctx + (j - lo)];
 #pragma unroll
