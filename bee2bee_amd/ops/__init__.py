@@ -511,8 +511,9 @@ def gqa_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
              cu_seqlens, softcap: float, talk, sink, head_gate, window: int,
              out, max_qlen: int = 0) -> None:
     """max_qlen: longest chunk of the step (host int). Without a cap and a
-    score mix the step runs on the sink-attention kernels (matrix cores for
-    bf16 prompt portions); with them, on the score-mixing kernels."""
+    score mix the step runs on the sink-attention kernels; with them, on
+    the score-mixing kernels. Both take bf16 prompt portions with head size
+    64/128 to the matrix cores."""
     if _use_hip(q):
         if talk is None and not softcap:
             require_hip().sink_attn(q, k_cache, v_cache, block_table,
@@ -523,8 +524,9 @@ def gqa_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
                 talk = torch.eye(q.shape[1], dtype=torch.float32,
                                  device=q.device)
             require_hip().mixed_score_attn(q, k_cache, v_cache, block_table,
-                                           positions, seq_idx, float(softcap),
-                                           talk, sink, head_gate, window, out)
+                                           positions, seq_idx, cu_seqlens,
+                                           float(softcap), talk, sink,
+                                           head_gate, window, out, max_qlen)
         return
     reference.gqa_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
                        cu_seqlens, softcap, talk, sink, head_gate, window, out)

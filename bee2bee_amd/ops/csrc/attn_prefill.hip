@@ -142,7 +142,18 @@ __global__ __launch_bounds__(64) void attn_prefill_basic(
 // p sees keys p - window < j <= p, and key tiles wholly before the tile's
 // first window are skipped. head_gate (optional, bf16 [tokens, nq] with row
 // stride s_g): head h's output times sigmoid(head_gate[t, h]).
-template <int HD, bool PAGED, typename KVT, bool HILO = false>
+//
+// MODE 1 / MODE 2 split the kernel around a score buffer, for attention
+// whose scores are mixed across heads before the softmax: MODE 1 stops
+// after S = Q K^T, caps it (softcap > 0: softcap * tanh(s / softcap)) and
+// writes the tile — masked entries too, as they come — to score_buf; MODE
+// 2 takes its score tiles from score_buf instead of computing them (another
+// kernel has mixed the heads in between) and goes on with mask, softmax,
+// P V and the epilogue. score_buf [nseq, qt_rows, nq, ctx] fp32 holds the
+// query rows [qt0 * 64, qt0 * 64 + qt_rows) of every chunk; entry `col` of
+// a row is key kv_lo + col, kv_lo being the first key the row's 64-query
+// tile visits. blockIdx.x counts tiles from qt0.
+template <int HD, bool PAGED, typename KVT, bool HILO = false, int MODE = 0>
 __global__ __launch_bounds__(256) void attn_prefill_mfma(
     const unsigned short* __restrict__ q,
     const KVT* __restrict__ k,  // PAGED: k_cache [nb,nkv,bs,hd]
@@ -154,7 +165,8 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
     int nq, int nkv, long s_q, long s_k, long s_v, int W, int bs,
     float scale, const float* __restrict__ sink, float out_scale, long s_o,
     int window = 0, const unsigned short* __restrict__ head_gate = nullptr,
-    long s_g = 0) {
+    long s_g = 0, float* __restrict__ score_buf = nullptr, int qt0 = 0,
+    int qt_rows = 0, long ctx = 0, float softcap = 0.f) {
     constexpr int KSTEPS = HD / 32;
     const int seq = blockIdx.z;
     const int h = blockIdx.y;
@@ -164,7 +176,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
     const int L = PAGED ? seq_lens[seq] : QL;  // keys incl. cached history
     const int hist = L - QL;
     const int* bt = PAGED ? block_table + (long)seq * W : nullptr;
-    const int q0 = blockIdx.x * PF_TM;  // q tile base (chunk-local row)
+    const int q0 = (blockIdx.x + qt0) * PF_TM;  // q tile base (chunk-local row)
     if (q0 >= QL) return;
 
     const int tid = threadIdx.x;
@@ -190,7 +202,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
     bf16x8 a_q[KSTEPS];
     const int my_qrow = q0 + wid * PF_QROWS + li;  // A row = li
     const bool row_ok = my_qrow < QL;
-    {
+    if (MODE != 2) {
         const unsigned short* qr = q + (long)(s0 + my_qrow) * s_q + (long)h * HD;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
@@ -238,8 +250,8 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
                     if (PAGED) {
                         const long koff = (((long)bt[gk / bs] * nkv + kvh) *
                                            bs + gk % bs) * HD + d;
-                        kraw = load_kv8_bf16(k + koff);
-                        vraw = load_kv8_bf16(v + koff);
+                        if (MODE != 2) kraw = load_kv8_bf16(k + koff);
+                        if (MODE != 1) vraw = load_kv8_bf16(v + koff);
                     } else {
                         kraw = load_kv8_bf16(
                             k + (long)(s0 + gk) * s_k + (long)kvh * HD + d);
@@ -247,29 +259,65 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
                             v + (long)(s0 + gk) * s_v + (long)kvh * HD + d);
                     }
                 }
-                *reinterpret_cast<bf16x8*>(k_s + key * (HD + PF_PAD) + d) = kraw;
+                if (MODE != 2)
+                    *reinterpret_cast<bf16x8*>(k_s + key * (HD + PF_PAD) + d) =
+                        kraw;
+                if (MODE != 1) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    vt_s[(d + e) * VT_STRIDE + key] =
-                        ((const unsigned short*)&vraw)[e];
+                    for (int e = 0; e < 8; ++e)
+                        vt_s[(d + e) * VT_STRIDE + key] =
+                            ((const unsigned short*)&vraw)[e];
+                }
             }
         }
         __syncthreads();
 
         // ---- S = Q K^T : PF_TN/16 16-key column fragments
         f32x4 sfrag[PF_TN / 16];
+        if (MODE == 2) {
+            // the (head-mixed) scores of this tile, C layout: col li, rows
+            // lg*4 + r
 #pragma unroll
-        for (int f = 0; f < PF_TN / 16; ++f) {
-            f32x4 acc{0.f, 0.f, 0.f, 0.f};
+            for (int f = 0; f < PF_TN / 16; ++f)
 #pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) {
-                // B-frag: col = key (li + 16f), k = dim ks*32 + lg*8 + e
-                bf16x8 bk = *reinterpret_cast<const bf16x8*>(
-                    k_s + (f * 16 + li) * (HD + PF_PAD) + ks * 32 + lg * 8);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_q[ks], bk, acc,
-                                                              0, 0, 0);
+                for (int r = 0; r < 4; ++r) {
+                    const int qrow = q0 + wid * PF_QROWS + lg * 4 + r;
+                    float sv = 0.f;
+                    if (qrow < QL)
+                        sv = score_buf[(((long)seq * qt_rows +
+                                         (qrow - qt0 * PF_TM)) * nq + h) * ctx +
+                                       (kb - kv_lo + f * 16 + li)];
+                    sfrag[f][r] = sv;
+                }
+        } else {
+#pragma unroll
+            for (int f = 0; f < PF_TN / 16; ++f) {
+                f32x4 acc{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ++ks) {
+                    // B-frag: col = key (li + 16f), k = dim ks*32 + lg*8 + e
+                    bf16x8 bk = *reinterpret_cast<const bf16x8*>(
+                        k_s + (f * 16 + li) * (HD + PF_PAD) + ks * 32 + lg * 8);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        a_q[ks], bk, acc, 0, 0, 0);
+                }
+                sfrag[f] = acc;
             }
-            sfrag[f] = acc;
+        }
+        if (MODE == 1) {
+#pragma unroll
+            for (int f = 0; f < PF_TN / 16; ++f)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int qrow = q0 + wid * PF_QROWS + lg * 4 + r;
+                    float sv = sfrag[f][r];
+                    if (softcap > 0.f) sv = softcap * tanhf(sv / softcap);
+                    if (qrow < QL)
+                        score_buf[(((long)seq * qt_rows +
+                                    (qrow - qt0 * PF_TM)) * nq + h) * ctx +
+                                  (kb - kv_lo + f * 16 + li)] = sv;
+                }
+            continue;       // the barrier at the loop head guards k_s
         }
 
         // ---- causal mask + online softmax (rows rr = lg*4 + r)
@@ -364,6 +412,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
         }
     }
 
+    if (MODE == 1) return;
     // ---- epilogue: normalize and store (C layout: col=li, row=lg*4+r)
     const int orow_base = q0 + wid * PF_QROWS;
 #pragma unroll
@@ -496,6 +545,84 @@ extern "C" int launch_attn_prefill_paged_sink(
             dim3(256), smem, stream, q, k_cache, v_cache, cu, block_table,
             seq_lens, out, nq, nkv, s_q, 0, 0, W, bs, 1.f, sink, out_scale,
             s_o, window, head_gate, s_g);
+    return 0;
+}
+
+// ------------------------------------------------- scores mixed across heads
+// In place on a score buffer [nseq, qt_rows, nq, ctx] (see attn_prefill_mfma
+// MODE 1/2): s'_h = sum_g mix[h, g] s_g at every (row, column) the tile
+// kernels visit. Workgroup = SM_ROWS rows x 64 columns; a thread stages the
+// nq scores of its (row, column) in LDS, then writes the nq mixtures back to
+// the same places (it is their only reader and writer).
+constexpr int SM_ROWS = 4;
+__global__ __launch_bounds__(64 * SM_ROWS) void score_mix_kernel(
+    float* __restrict__ score_buf, const float* __restrict__ mix,
+    const int* __restrict__ cu, const int* __restrict__ seq_lens, int nq,
+    int qt0, int qt_rows, long ctx, int window) {
+    extern __shared__ __attribute__((aligned(16))) float sm_s[];
+    float* tk = sm_s;                              // [nq, nq]
+    float* col = sm_s + nq * nq + threadIdx.x;     // [nq] at stride blockDim
+    for (int i = threadIdx.x; i < nq * nq; i += blockDim.x) tk[i] = mix[i];
+    __syncthreads();
+    const int seq = blockIdx.z;
+    const int lr = blockIdx.y * SM_ROWS + threadIdx.x / 64;
+    const int c = blockIdx.x * 64 + threadIdx.x % 64;
+    if (lr >= qt_rows) return;
+    const int s0 = cu[seq], QL = cu[seq + 1] - s0;
+    const int qrow = qt0 * PF_TM + lr;
+    if (qrow >= QL) return;
+    const int L = seq_lens[seq], hist = L - QL;
+    const int q0 = qrow / PF_TM * PF_TM;
+    const int kv_end = min(L, hist + q0 + PF_TM);
+    const int kv_lo =
+        window > 0 ? max(0, hist + q0 - window + 1) / PF_TN * PF_TN : 0;
+    if (c >= (kv_end - kv_lo + PF_TN - 1) / PF_TN * PF_TN) return;
+    float* p = score_buf + ((long)seq * qt_rows + lr) * nq * ctx + c;
+    const int st = blockDim.x;
+    for (int g = 0; g < nq; ++g) col[g * st] = p[(long)g * ctx];
+    for (int h = 0; h < nq; ++h) {
+        float a = 0.f;
+        for (int g = 0; g < nq; ++g) a += tk[h * nq + g] * col[g * st];
+        p[(long)h * ctx] = a;
+    }
+}
+
+// Packed query chunks against the paged history with capped scores mixed
+// across heads before the softmax: tile scores (MODE 1), the mix, then
+// softmax and P V from the mixed tiles (MODE 2; weights as a bf16 hi+lo
+// pair, sink and head gate in the epilogue). Covers the 64-query tiles
+// [qt0, qt0 + n_tiles) of every chunk; score_buf holds nseq * n_tiles * 64
+// * nq * ctx floats. bf16, head size 64 or 128 (nonzero otherwise); scale
+// is folded into q by the caller.
+extern "C" int launch_attn_prefill_paged_mixed(
+    const unsigned short* q, long s_q, const unsigned short* k_cache,
+    const unsigned short* v_cache, const int* cu, const int* block_table,
+    const int* seq_lens, unsigned short* out, long s_o, int nseq, int nq,
+    int nkv, int hd, int W, int bs, int qt0, int n_tiles, float* score_buf,
+    long ctx, float softcap, const float* mix, const float* sink, int window,
+    const unsigned short* head_gate, long s_g, hipStream_t stream) {
+    if (hd != 64 && hd != 128) return 1;
+    if (nseq == 0 || n_tiles == 0) return 0;
+    const int qt_rows = n_tiles * PF_TM;
+    const dim3 grid(n_tiles, nq, nseq);
+    const int smem = prefill_mfma_smem(hd, 1);
+    const size_t mix_smem =
+        ((size_t)nq * nq + (size_t)nq * 64 * SM_ROWS) * sizeof(float);
+    if (mix_smem > 64 * 1024) return 1;
+    const dim3 mgrid((unsigned)((ctx + 63) / 64),
+                     (qt_rows + SM_ROWS - 1) / SM_ROWS, nseq);
+#define PM_LAUNCH(HDV, M)                                                     \
+    hipLaunchKernelGGL(                                                       \
+        (attn_prefill_mfma<HDV, true, unsigned short, true, M>), grid,        \
+        dim3(256), smem, stream, q, k_cache, v_cache, cu, block_table,        \
+        seq_lens, out, nq, nkv, s_q, 0, 0, W, bs, 1.f, sink, 1.f, s_o,        \
+        window, head_gate, s_g, score_buf, qt0, qt_rows, ctx, softcap)
+    if (hd == 128) PM_LAUNCH(128, 1); else PM_LAUNCH(64, 1);
+    hipLaunchKernelGGL(score_mix_kernel, mgrid, dim3(64 * SM_ROWS), mix_smem,
+                       stream, score_buf, mix, cu, seq_lens, nq, qt0, qt_rows,
+                       ctx, window);
+    if (hd == 128) PM_LAUNCH(128, 2); else PM_LAUNCH(64, 2);
+#undef PM_LAUNCH
     return 0;
 }
 

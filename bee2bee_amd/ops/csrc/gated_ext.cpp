@@ -37,6 +37,11 @@ int launch_mixed_score_attn(const void*, long, const void*, const void*,
                             void*, long, float*, long, float*, float*, float*,
                             int, int, int, int, int, int, int, int, int,
                             hipStream_t);
+int launch_attn_prefill_paged_mixed(
+    const unsigned short*, long, const unsigned short*, const unsigned short*,
+    const int*, const int*, const int*, unsigned short*, long, int, int, int,
+    int, int, int, int, int, float*, long, float, const float*, const float*,
+    int, const unsigned short*, long, hipStream_t);
 }
 
 namespace {
@@ -292,13 +297,17 @@ void min_gru(const Tensor& z, const Tensor& x, const Tensor& g, Tensor& state,
 // Grouped-query attention whose capped scores are mixed across heads before
 // the softmax. The scores of a block of rows are written once ([rows, H,
 // ctx] fp32, at most ~256 MB per block; longer steps run block by block).
+// bf16 prompt portions (max_qlen >= 16) with head size 64/128 run on the
+// matrix cores: tile scores, the mix, then softmax and P V from the mixed
+// tiles; fp32, other head sizes and decode steps take the wave-per-row
+// kernels.
 void mixed_score_attn(const Tensor& q, const Tensor& k_cache,
                       const Tensor& v_cache, const Tensor& block_table,
                       const Tensor& positions, const Tensor& seq_idx,
-                      double softcap, const Tensor& mix,
+                      const Tensor& cu, double softcap, const Tensor& mix,
                       const std::optional<Tensor>& sink,
                       const std::optional<Tensor>& head_gate, int64_t window,
-                      Tensor& out) {
+                      Tensor& out, int64_t max_qlen) {
     const int c = act_code(q, "q");
     check_i32(block_table, "block_table");
     check_i32(positions, "positions");
@@ -335,8 +344,45 @@ void mixed_score_attn(const Tensor& q, const Tensor& k_cache,
         hg_tok = head_gate->stride(0);
     }
     if (Tn == 0) return;
+    check_i32(cu, "cu_seqlens");
     // the most keys a row can see, in whole 64-key tiles
     const long reach = block_table.size(1) * (long)bs;
+    auto f32opt = q.options().dtype(torch::kFloat32);
+    if (c == 0 && max_qlen >= 16 && D == Dv && (D == 64 || D == 128) &&
+        (size_t)H * H * 4 + (size_t)H * 1024 <= 64 * 1024) {
+        const long B = cu.numel() - 1;
+        TORCH_CHECK(block_table.size(0) == B);
+        Tensor last = cu.slice(0, 1, B + 1).to(torch::kLong) - 1;
+        Tensor seq_lens =
+            (positions.index_select(0, last.clamp_min(0)) + 1)
+                .to(torch::kInt32);
+        // a 64-query tile visits at most window + 126 keys, in 64-key tiles
+        long tctx = window > 0 ? std::min<long>(window + 128, reach + 64)
+                               : reach + 64;
+        tctx = (tctx + 63) / 64 * 64;
+        const long tiles = (max_qlen + 63) / 64;
+        // tiles per launch: a score buffer of at most ~256 MB
+        const long per =
+            std::max<long>(1, (64L << 20) / (B * 64 * H * tctx));
+        const long nt = std::min<long>(tiles, per);
+        Tensor buf = torch::empty({B, nt * 64, (long)H, tctx}, f32opt);
+        for (long t0 = 0; t0 < tiles; t0 += nt) {
+            const int rc = launch_attn_prefill_paged_mixed(
+                (const unsigned short*)q.data_ptr(), q.stride(0),
+                (const unsigned short*)k_cache.data_ptr(),
+                (const unsigned short*)v_cache.data_ptr(),
+                cu.data_ptr<int>(), block_table.data_ptr<int>(),
+                seq_lens.data_ptr<int>(), (unsigned short*)out.data_ptr(),
+                out.stride(0), (int)B, H, G, D, (int)block_table.size(1), bs,
+                (int)t0, (int)std::min<long>(nt, tiles - t0),
+                buf.data_ptr<float>(), tctx, (float)softcap,
+                mix.data_ptr<float>(), sk, (int)window,
+                (const unsigned short*)hg, hg_tok, stream());
+            TORCH_CHECK(rc == 0, "mixed_score_attn: matrix-core path refused "
+                                 "a shape its guard admitted");
+        }
+        return;
+    }
     long ctx = window > 0 ? std::min<long>(window, reach) : reach;
     ctx = (ctx + 63) / 64 * 64;
     const long block_rows = std::max<long>(
@@ -346,7 +392,6 @@ void mixed_score_attn(const Tensor& q, const Tensor& k_cache,
     long splits = 8192 / std::max<long>(1, block_rows * units);
     splits = std::min<long>({splits, 32, (ctx + 63) / 64});
     splits = std::max<long>(splits, 1);
-    auto f32opt = q.options().dtype(torch::kFloat32);
     Tensor scores = torch::empty({block_rows, (long)H, ctx}, f32opt);
     Tensor scratch = torch::empty({splits, block_rows, (long)H, 2}, f32opt);
     Tensor part_acc, part_ml;

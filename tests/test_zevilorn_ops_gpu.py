@@ -218,6 +218,29 @@ def test_plain_attention_matrix_core_windows(D, G, window, sink, gated):
     torch.testing.assert_close(a, b, rtol=2e-2, atol=4e-2)
 
 
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("G,window", [(1, 0), (2, 100), (4, 64), (2, 1),
+                                      (3, 300), (2, 40), (2, 65)])
+@pytest.mark.parametrize("softcap,sink,gated", [(3.0, "zero", False),
+                                                (0.0, "learned", True)])
+def test_mixed_score_attention_matrix_core(D, G, window, softcap, sink, gated):
+    """bf16 prompt portions of head size 64/128: tile scores on the matrix
+    cores, the head mix on the score buffer, softmax and P V from the mixed
+    tiles; windows that end inside, at and before a key tile, chunks with
+    history, a chunk shorter than a tile, single rows riding along"""
+    a, b = _gqa_case(torch.bfloat16, [70, 1, 130, 16, 1],
+                     [0, 200, 57, 500, 0], 2 * G, G, D, D, window, 32,
+                     softcap, True, sink, gated, seed=3)
+    torch.testing.assert_close(a, b, rtol=2e-2, atol=4e-2)
+
+
+def test_mixed_score_attention_matrix_core_many_tiles():
+    """a long portion cut into several launches of the score buffer"""
+    a, b = _gqa_case(torch.bfloat16, [700, 300], [100, 0], 8, 2, 64, 64, 0,
+                     64, 2.0, True, "zero", False, seed=4)
+    torch.testing.assert_close(a, b, rtol=2e-2, atol=4e-2)
+
+
 def _latent_case(dtype, lens, starts, H, C, R, window, sink, bs=16, seed=3):
     torch.manual_seed(seed)
     need = sum(-(-(s + L) // bs) for L, s in zip(lens, starts))
