@@ -142,13 +142,14 @@ def test_graph_decode_equals_eager(tmp_path):
 @pytest.mark.parametrize("left_kv,left_window", [(2, 50), (4, 0)])
 def test_head_sizes_of_the_matrix_core_paths(tmp_path, dtype, left_kv,
                                              left_window):
-    """Heads of 64 in the windowed attention and a latent row of 64 + 32:
+    """Heads of 64 in both grouped-query attentions (score-mixing and
+    windowed) and a latent row of 64 + 32:
     bf16 prompt portions of 16 tokens or more run on the matrix cores,
     shorter portions and decode rows on the generic kernels with their key
     splits; fp32 takes the generic kernels throughout. All must agree with
     the oracle on one sequence cut in different ways."""
     cfg = O.make_config(width=64, vocab=90, ff=24, heads=4, kv_heads=2,
-                        dim=32, vdim=32, rot_dims=32, window=70,
+                        dim=64, vdim=64, rot_dims=32, window=70,
                         lat_heads=4, lat_dim=16, rot_dim=32, lat_vdim=16,
                         kv_rank=64, q_rank=24, left_heads=4, left_kv=left_kv,
                         left_dim=64, left_vdim=64, left_window=left_window,
@@ -165,3 +166,22 @@ def test_head_sizes_of_the_matrix_core_paths(tmp_path, dtype, left_kv,
                   [[("a", 170)]] + [[("a", 1)]] * 40):
         got = replay(eng, {"a": toks}, sched)["a"]
         assert_logits(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_expert_execution_strategies(tmp_path, dtype):
+    """Steps of 300 and 700 tokens at a width and expert size the
+    grouped-GEMM kernel covers (bf16: sorted token slots through the kernel;
+    beyond its range and in fp32 the per-expert loop), decode rows through
+    the dense all-experts product: all equal the oracle."""
+    cfg = O.make_config(width=128, vocab=80, ff=128, experts=8, top=2,
+                        n_groups=4, keep=2, kinds=("parallel", "attention"),
+                        loop=None, gru=24)
+    W = O.random_weights(cfg, seed=26)
+    eng = make_engine(tmp_path, cfg, W, device="cuda", dtype=dtype,
+                      kv_blocks=80)
+    toks = random_tokens(1010, cfg["vocab"], 12)
+    want = oracle_logits(cfg, W, toks)
+    got = replay(eng, {"a": toks},
+                 [[("a", 300)], [("a", 700)]] + [[("a", 1)]] * 10)["a"]
+    assert_logits(got, want, dtype)
