@@ -484,7 +484,15 @@ def silu_glu(gate_up):
 
 def group_topk_gate(logits, top_k: int, n_groups: int, keep_groups: int,
                     score: str = "softmax", group_top: int = 1):
-    # [T, E] gating math: torch ops on both devices, like moe_topk_gate
+    """One kernel on the GPU (a thread per token, scores in LDS) while the
+    experts of a workgroup's tokens fit; torch ops otherwise and on the
+    CPU."""
+    E = logits.shape[1]
+    if _use_hip(logits) and (E + n_groups) * 256 <= 64 * 1024:
+        w, idx = require_hip().group_topk_gate(
+            logits.float().contiguous(), top_k, n_groups, keep_groups,
+            score == "sigmoid", group_top)
+        return w, idx
     return reference.group_topk_gate(logits, top_k, n_groups, keep_groups,
                                      score, group_top)
 

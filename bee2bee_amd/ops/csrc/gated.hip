@@ -395,6 +395,85 @@ min_gru_scan_kernel(const int* __restrict__ cu,
     *st = S;
 }
 
+// ------------------------------------------------ group-limited routing
+// One thread per token; its E scores (and group scores) live in LDS at
+// stride blockDim, so neighbouring threads never share a bank. scores =
+// sigmoid(logit) or softmax over all experts; a group's score is the sum of
+// its group_top largest scores; experts outside the best `keep` groups
+// cannot be chosen; the top_k best remaining scores are the weights, as they
+// are, in descending order (ties: the lower index first).
+constexpr int GT_THREADS = 64;
+__global__ void __launch_bounds__(GT_THREADS)
+group_topk_gate_kernel(const float* __restrict__ logits,
+                       float* __restrict__ w_out, int* __restrict__ idx_out,
+                       long T, int E, int top_k, int n_groups, int keep,
+                       int group_top, int sigmoid) {
+    extern __shared__ __attribute__((aligned(16))) float gt_s[];
+    const long t = (long)blockIdx.x * GT_THREADS + threadIdx.x;
+    if (t >= T) return;                    // no workgroup barrier below
+    float* sc = gt_s + threadIdx.x;                       // [E]
+    float* gsc = gt_s + (long)E * GT_THREADS + threadIdx.x;  // [n_groups]
+    const int st = GT_THREADS;
+    const float* z = logits + t * E;
+    if (sigmoid) {
+        for (int e = 0; e < E; ++e) sc[e * st] = sigmoid_f(z[e]);
+    } else {
+        float m = -INFINITY, sum = 0.f;
+        for (int e = 0; e < E; ++e) m = fmaxf(m, z[e]);
+        for (int e = 0; e < E; ++e) {
+            const float x = expf(z[e] - m);
+            sc[e * st] = x;
+            sum += x;
+        }
+        for (int e = 0; e < E; ++e) sc[e * st] /= sum;
+    }
+    const int gs = E / n_groups;
+    const bool limited = n_groups > 1 && keep < n_groups;
+    if (limited) {
+        const int gt = min(max(group_top, 1), gs);
+        for (int g = 0; g < n_groups; ++g) {
+            // sum of the gt largest: each pass takes the largest score that
+            // is below the last one taken (or equal, at a higher index)
+            float total = 0.f, last = INFINITY;
+            int last_i = -1;
+            for (int it = 0; it < gt; ++it) {
+                float best = -1.f;
+                int bi = -1;
+                for (int j = 0; j < gs; ++j) {
+                    const float x = sc[(g * gs + j) * st];
+                    const bool open = x < last || (x == last && j > last_i);
+                    if (open && x > best) { best = x; bi = j; }
+                }
+                total += best;
+                last = best;
+                last_i = bi;
+            }
+            gsc[g * st] = total;
+        }
+        for (int it = 0; it < keep; ++it) {
+            float best = -1.f;
+            int bg = 0;
+            for (int g = 0; g < n_groups; ++g) {
+                const float x = gsc[g * st];
+                if (x > best) { best = x; bg = g; }
+            }
+            gsc[bg * st] = -2.f;           // kept
+        }
+    }
+    for (int it = 0; it < top_k; ++it) {
+        float best = -1.f;
+        int be = 0;
+        for (int e = 0; e < E; ++e) {
+            if (limited && gsc[(e / gs) * st] != -2.f) continue;
+            const float x = sc[e * st];
+            if (x > best) { best = x; be = e; }
+        }
+        w_out[t * top_k + it] = best;
+        idx_out[t * top_k + it] = be;
+        sc[be * st] = -1.f;                // taken
+    }
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------- launchers
@@ -532,4 +611,19 @@ extern "C" void launch_min_gru(const void* z, long zs, const void* x, long xs,
     if (c) MG_SEG_LAUNCH(float, 3);
     else MG_SEG_LAUNCH(unsigned short, 3);
 #undef MG_SEG_LAUNCH
+}
+
+// Returns nonzero when the scores of a workgroup's tokens do not fit LDS.
+extern "C" int launch_group_topk_gate(const float* logits, float* w_out,
+                                      int* idx_out, long T, int E, int top_k,
+                                      int n_groups, int keep, int group_top,
+                                      int sigmoid, hipStream_t s) {
+    const size_t smem = (size_t)(E + n_groups) * GT_THREADS * sizeof(float);
+    if (smem > 64 * 1024) return 1;
+    if (T == 0) return 0;
+    const unsigned grid = (unsigned)((T + GT_THREADS - 1) / GT_THREADS);
+    group_topk_gate_kernel<<<grid, GT_THREADS, smem, s>>>(
+        logits, w_out, idx_out, T, E, top_k, n_groups, keep, group_top,
+        sigmoid);
+    return 0;
 }

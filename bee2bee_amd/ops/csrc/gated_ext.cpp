@@ -9,6 +9,7 @@
 
 #include <algorithm>
 #include <optional>
+#include <vector>
 
 using torch::Tensor;
 
@@ -37,6 +38,8 @@ int launch_mixed_score_attn(const void*, long, const void*, const void*,
                             void*, long, float*, long, float*, float*, float*,
                             int, int, int, int, int, int, int, int, int,
                             hipStream_t);
+int launch_group_topk_gate(const float*, float*, int*, long, int, int, int,
+                           int, int, int, hipStream_t);
 int launch_attn_prefill_paged_mixed(
     const unsigned short*, long, const unsigned short*, const unsigned short*,
     const int*, const int*, const int*, unsigned short*, long, int, int, int,
@@ -420,9 +423,35 @@ void mixed_score_attn(const Tensor& q, const Tensor& k_cache,
     }
 }
 
+std::vector<Tensor> group_topk_gate(const Tensor& logits, int64_t top_k,
+                                    int64_t n_groups, int64_t keep,
+                                    bool sigmoid, int64_t group_top) {
+    check_f32(logits, "logits");
+    TORCH_CHECK(logits.dim() == 2);
+    const long T = logits.size(0);
+    const int E = (int)logits.size(1);
+    TORCH_CHECK(n_groups >= 1 && E % n_groups == 0 && keep >= 1 &&
+                keep <= n_groups && top_k >= 1 &&
+                top_k <= keep * (E / n_groups),
+                "experts must split into equal groups and the kept groups "
+                "must hold top_k experts");
+    Tensor w = torch::empty({T, top_k}, logits.options());
+    Tensor idx = torch::empty({T, top_k},
+                              logits.options().dtype(torch::kInt32));
+    const int rc = launch_group_topk_gate(
+        logits.data_ptr<float>(), w.data_ptr<float>(), idx.data_ptr<int>(), T,
+        E, (int)top_k, (int)n_groups, (int)keep, (int)group_top,
+        sigmoid ? 1 : 0, stream());
+    TORCH_CHECK(rc == 0, "group_topk_gate: too many experts for one "
+                         "workgroup's LDS");
+    return {w, idx};
+}
+
 }  // namespace
 
 void register_gated_ops(pybind11::module_& m) {
+    m.def("group_topk_gate", &group_topk_gate,
+          "group-limited expert choice on sigmoid or softmax scores");
     m.def("gated_add_rmsnorm", &gated_add_rmsnorm,
           "resid += sigmoid(g1) y1 [+ sigmoid(g2) y2] [+ extra]; "
           "out = unit(resid) * w");

@@ -272,3 +272,21 @@ def test_latent_attention_sink(dtype, H, C, R, window, sink):
                          ([1, 1, 1, 1, 1], [0, 47, 15, 200, 95])):
         a, b = _latent_case(dtype, lens, starts, H, C, R, window, sink)
         torch.testing.assert_close(a, b, **tol(dtype))
+
+
+@pytest.mark.parametrize("score", ["sigmoid", "softmax"])
+@pytest.mark.parametrize("E,top,n_groups,keep,group_top", [
+    (8, 3, 4, 3, 2), (8, 2, 2, 1, 2), (6, 1, 3, 2, 1), (4, 4, 1, 1, 1),
+    (9, 2, 9, 4, 1), (12, 3, 3, 3, 2), (64, 8, 8, 4, 2), (128, 6, 16, 3, 3)])
+def test_group_topk_gate(score, E, top, n_groups, keep, group_top):
+    """the routing kernel against the torch-op reference: same experts,
+    same weights (random logits have no ties)"""
+    torch.manual_seed(9)
+    logits = torch.randn(333, E, device=DEV) * 2
+    w1, i1 = ops.group_topk_gate(logits, top, n_groups, keep, score, group_top)
+    w2, i2 = ref.group_topk_gate(logits, top, n_groups, keep, score, group_top)
+    assert i1.dtype == torch.int32 and w1.dtype == torch.float32
+    o1, o2 = i1.long().sort(1), i2.long().sort(1)
+    assert torch.equal(o1.values, o2.values)
+    torch.testing.assert_close(w1.gather(1, o1.indices),
+                               w2.gather(1, o2.indices), rtol=1e-5, atol=1e-6)
