@@ -326,6 +326,41 @@ def test_latent_attention_with_sink_in_portions(sink, sched):
     assert torch.allclose(got.double(), want, atol=3e-5)
 
 
+@pytest.mark.parametrize("j", [0, 15, 16, 17, 131])
+@pytest.mark.parametrize("sched", [[300], [280] + [1] * 20])
+def test_latent_far_key_among_hundreds(j, sched):
+    """no window: one key far back — the first token, both sides of a page
+    border — dominates among 300; every later row returns its latent row,
+    in a prompt and in decoding, whatever the sink holds"""
+    torch.manual_seed(9)
+    H, C, R, T, bs = 2, 6, 2, 300, 16
+    lat = torch.randn(T, C) * 0.05
+    lat[j] = torch.tensor([4.0, -3.0, 2.0, 1.0, -2.0, 3.0])
+    m = pages([T], [0], bs)
+    cache = torch.full((m["nb"], bs, C + R), float("nan"))
+    flat = cache.view(-1, C + R)
+    flat[m["slot"].long()] = torch.cat([lat, torch.zeros(T, R)], -1)
+    # every query points along the planted row
+    q_abs = (lat[j] * 3.0).expand(H, T, C).contiguous()
+    q_rot = torch.zeros(T, H, R)
+    gate = torch.full((T, H), 40.0)
+    sk = torch.tensor([1.0, -2.0])
+    got, at = [], 0
+    for n in sched:
+        pos = i32(list(range(at, at + n)))
+        got.append(ref.latent_attn(q_abs[:, at:at + n].contiguous(),
+                                   q_rot[at:at + n], gate[at:at + n], cache,
+                                   m["bt"], pos, i32([0] * n), i32([0, n]), 0,
+                                   1.0, sink=sk))
+        at += n
+    got = torch.cat(got, 1)
+    for t in (max(j, 1), j + 1, 299):
+        if t >= j:
+            assert torch.allclose(got[:, t], lat[j].expand(H, C), atol=1e-3), t
+    if j > 0:       # rows before it do not see it
+        assert float(got[:, j - 1].abs().max()) < 1.0
+
+
 def test_latent_sink_is_not_scaled_and_counts_once():
     """all scores equal: the sink's share is e^sink / (e^sink + n e^s)"""
     H, C, R, T = 2, 3, 2, 5
