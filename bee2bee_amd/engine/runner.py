@@ -51,6 +51,7 @@ class Runner:
         # attention layers, and an optional per-layer probe
         # layer_tap(layer_idx, residual_fp32) for bring-up/debugging
         self._rope_by_cfg = {}
+        self._zeros = {}        # fp32 zero vectors by length (zero-logit sinks)
         self.layer_tap = None
         if spec.is_hybrid:
             self.rope_cos = self.rope_sin = None
@@ -763,10 +764,10 @@ class Runner:
         return out
 
     def _zeros_f32(self, n: int) -> torch.Tensor:
-        z = self._rope_by_cfg.get(("zeros", n))
+        z = self._zeros.get(n)
         if z is None:
-            z = self._rope_by_cfg[("zeros", n)] = torch.zeros(
-                n, dtype=torch.float32, device=self.device)
+            z = self._zeros[n] = torch.zeros(n, dtype=torch.float32,
+                                             device=self.device)
         return z
 
     def _latent_attn_part(self, i: int, m, ns, cols, pre, meta
